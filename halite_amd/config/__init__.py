@@ -1,4 +1,5 @@
 from .engine import ModelConfig, ServerConfig, parse_overrides
+from .kavuvik import KavuvikConfig
 from .model import Llama3RopeScaling, LlamaConfig
 from .registry import (
     ARCHITECTURES,
@@ -15,6 +16,7 @@ __all__ = [
     "ARCHITECTURES",
     "Architecture",
     "ConfigError",
+    "KavuvikConfig",
     "LayerRun",
     "LayerSpec",
     "Llama3RopeScaling",

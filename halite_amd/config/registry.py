@@ -31,7 +31,8 @@ class Architecture:
     ``config_cls`` is a pydantic model of the architecture's ``config.json``.  Beside its
     own keys it must have the field ``architectures`` (a list whose first entry is
     ``name``: what a model folder is recognised by, and what the random-weights mode
-    writes).  It may have ``stop_token_ids`` (token ids that end a request unless it asks
+    writes; a file that names its architecture as a string under ``architecture`` has that
+    field and a property ``architectures`` instead).  It may have ``stop_token_ids`` (token ids that end a request unless it asks
     to ignore them) and a method ``to_json_dict()`` (the ``config.json`` to write, if
     ``model_dump(exclude_none=True)`` is not it).  Nothing else of it is read outside
     ``to_spec`` and ``weight_map``, which are the architecture's own."""
@@ -49,10 +50,11 @@ ARCHITECTURES: dict[str, Architecture] = {}
 
 def register_architecture(arch: Architecture) -> Architecture:
     fields = getattr(arch.config_cls, "model_fields", None)
-    if fields is None or "architectures" not in fields:
+    if fields is None or ("architectures" not in fields and not isinstance(getattr(arch.config_cls, "architectures", None), property)):
         raise ConfigError(
             f"architecture {arch.name!r}: its configuration class must be a pydantic model with "
-            "the field 'architectures'"
+            "the field 'architectures' (or, where the file names its one architecture under "
+            "'architecture', with that field and a property 'architectures')"
         )
     for optional in ("to_json_dict",):
         if hasattr(arch.config_cls, optional) and not callable(getattr(arch.config_cls, optional)):
@@ -75,8 +77,10 @@ def _load_builtin():
 
 def parse_config(raw: dict) -> tuple[Architecture, BaseModel]:
     names = raw.get("architectures")
+    if names is None and isinstance(raw.get("architecture"), str):
+        names = [raw["architecture"]]  # a file that names its one architecture as a string
     if not names or not isinstance(names, list):
-        raise ConfigError("config.json has no 'architectures' list")
+        raise ConfigError("config.json has no 'architectures' list (or 'architecture' name)")
     arch = get_architecture(names[0])
     try:
         cfg = arch.config_cls(**raw)

@@ -12,7 +12,7 @@
 // ---------------------------------------------------------------------------------
 template <typename TT>
 __global__ void embedding_kernel(const int* __restrict__ ids, const TT* __restrict__ table,
-                                 float* __restrict__ out, int d, int vocab) {
+                                 float* __restrict__ out, int d, int vocab, float scale) {
   const int t = blockIdx.x;
   const int id = ids[t];
   float* o = out + (size_t)t * d;
@@ -22,13 +22,13 @@ __global__ void embedding_kernel(const int* __restrict__ ids, const TT* __restri
     return;
   }
   const TT* row = table + (size_t)id * d;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = to_f32(row[i]);
+  for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = to_f32(row[i]) * scale;
 }
 
 // four elements per access; d is a multiple of 4
 template <typename TT>
 __global__ void embedding_vec_kernel(const int* __restrict__ ids, const TT* __restrict__ table,
-                                     float* __restrict__ out, int d, int vocab) {
+                                     float* __restrict__ out, int d, int vocab, float scale) {
   const int t = blockIdx.x;
   const int id = ids[t];
   float* o = out + (size_t)t * d;
@@ -37,6 +37,8 @@ __global__ void embedding_vec_kernel(const int* __restrict__ ids, const TT* __re
   for (int i = threadIdx.x * 4; i < d; i += blockDim.x * 4) {
     float v[4];
     load4(row + i, v);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] *= scale;
     if (!ok) v[0] = v[1] = v[2] = v[3] = __uint_as_float(0x7fc00000u);
     store4(o + i, v);
   }
@@ -63,6 +65,13 @@ extern "C" int hal_take_tokens(const int* src, int n_src, int* tokens, int n, hi
 
 extern "C" int hal_embedding(const int* ids, const void* table, int table_dtype, float* out,
                              int n_tokens, int d, int vocab, hipStream_t stream) {
+  return hal_embedding_scaled(ids, table, table_dtype, out, n_tokens, d, vocab, 1.0f, stream);
+}
+
+// the same with every row multiplied by `scale` (in float32)
+extern "C" int hal_embedding_scaled(const int* ids, const void* table, int table_dtype, float* out,
+                                    int n_tokens, int d, int vocab, float scale,
+                                    hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && d > 0 && vocab > 0, "hal_embedding: bad sizes T=%d d=%d V=%d",
               n_tokens, d, vocab);
   if (n_tokens == 0) return 0;
@@ -73,20 +82,20 @@ extern "C" int hal_embedding(const int* ids, const void* table, int table_dtype,
     if (threads > 1024) threads = 1024;
     if (table_dtype == HAL_F32)
       hipLaunchKernelGGL(embedding_vec_kernel<float>, dim3(n_tokens), dim3(threads), 0, stream,
-                         ids, (const float*)table, out, d, vocab);
+                         ids, (const float*)table, out, d, vocab, scale);
     else
       hipLaunchKernelGGL(embedding_vec_kernel<bf16_t>, dim3(n_tokens), dim3(threads), 0, stream,
-                         ids, (const bf16_t*)table, out, d, vocab);
+                         ids, (const bf16_t*)table, out, d, vocab, scale);
     HAL_LAUNCH_CHECK();
     return 0;
   }
   const int threads = d >= 1024 ? 256 : 64;
   if (table_dtype == HAL_F32)
     hipLaunchKernelGGL(embedding_kernel<float>, dim3(n_tokens), dim3(threads), 0, stream, ids,
-                       (const float*)table, out, d, vocab);
+                       (const float*)table, out, d, vocab, scale);
   else
     hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(n_tokens), dim3(threads), 0, stream, ids,
-                       (const bf16_t*)table, out, d, vocab);
+                       (const bf16_t*)table, out, d, vocab, scale);
   HAL_LAUNCH_CHECK();
   return 0;
 }

@@ -14,6 +14,10 @@ int hal_version();
 int hal_embedding(const int* ids, const void* table, int table_dtype, float* out, int n_tokens,
                   int d, int vocab, hipStream_t stream);
 
+// hal_embedding with every row multiplied by `scale` in float32.
+int hal_embedding_scaled(const int* ids, const void* table, int table_dtype, float* out,
+                         int n_tokens, int d, int vocab, float scale, hipStream_t stream);
+
 int hal_take_tokens(const int* src, int n_src, int* tokens, int n, hipStream_t stream);
 
 int hal_rmsnorm(float* h, const void* delta, const int* rows, const void* w, int w_dtype,
@@ -113,6 +117,59 @@ int hal_sample_spread(const float* logits, int ld, int n_rows, int V, const floa
                       const uint64_t* seeds, const int* draw_index, float* parts, float* kept,
                       void* state, void* hist, int any_late, int* out_token, float* out_logprob,
                       hipStream_t stream);
+
+// ---- products in groups (grouped_gemm.hip) ---------------------------------------------
+// Y_g = X_g * W_g^T for G groups in one launch, float32 accumulation; operands of `dtype`.
+// Group g reads the columns from g * x_group_cols + x_col0 of X's rows (row length ldx) and
+// W + g * w_group_stride ([N, K], row length ldw), and writes the columns from
+// g * y_group_cols + y_col0 of Y's rows (row length ldy, element type y_dtype; y_add: added
+// into a float32 Y).  group_offsets == null: every group has the rows 0 .. M-1.  Otherwise
+// group g has the rows group_offsets[g] .. group_offsets[g + 1] - 1 of a list of M rows in
+// all (tile_offsets: the same counted in tiles of 64 rows, each group rounded up; both
+// [G + 1] on the device): row i of the list reads row row_src[i] / src_div of X (i if null)
+// and writes row row_dst[i] of Y (i if null).  W2 != null: two products and the clamped
+// gated activation g = min(x W^T, limit), u = clamp(x W2^T, -limit, limit),
+// y = g * sigmoid(alpha * g) * (u + 1).  gate != null (float32 rows of length ldg): the
+// result is multiplied by sigmoid(gate[row, g * y_group_cols + n]).
+int hal_grouped_gemm(const void* X, int ldx, int x_group_cols, int x_col0, const void* W,
+                     const void* W2, long long w_group_stride, int ldw, int dtype, void* Y, int ldy,
+                     int y_group_cols, int y_col0, int y_dtype, int y_add, int M, int N, int K,
+                     int G, const int* group_offsets, const int* tile_offsets, const int* row_src,
+                     int src_div, const int* row_dst, const float* gate, int ldg, float limit,
+                     float alpha, int allow_mfma, hipStream_t stream);
+
+// ---- around a latent attention and a mixture of experts (latent_moe.hip) -----------------
+// RMSNorm of rows of the float32 stream (rows[r] or r) with one or two weights, x * rstd * w
+// in float32, rounded once.
+int hal_norm_pair(const float* h, const int* rows, const void* w1, const void* w2, int w_dtype,
+                  float eps, void* out1, void* out2, int dtype, int n_rows, int d,
+                  hipStream_t stream);
+// From the float32 down projections of a latent attention (a [T, lda]: query latent of q_rank
+// columns from q_col0, none if q_rank == 0; key/value latent of kv_rank columns from kv_col0
+// followed by `rot` shared rotated-key columns): cq [T, q_rank] = the normed query latent,
+// and in the packed rows qkv (row length row_stride) the key row [rot | normed latent | 0]
+// at column k_col0 and the value row [0 | normed latent | 0] at k_col0 + D, D columns each.
+int hal_latent_prep(const float* a, int lda, int q_col0, int q_rank, int kv_col0, int kv_rank,
+                    int rot, int D, const void* wq, const void* wkv, int w_dtype, float eps,
+                    void* cq, void* qkv, int row_stride, int k_col0, int dtype, int n_tokens,
+                    hipStream_t stream);
+// y[t, h * ys + y0 + j] = x[t, h * xs + x0 + j] (j < n) and zero in the n_zero columns from
+// h * ys + z0, for H heads.
+int hal_head_cols(const void* x, int ldx, int xs, int x0, void* y, int ldy, int ys, int y0, int n,
+                  int z0, int n_zero, int H, int dtype, int n_tokens, hipStream_t stream);
+int hal_scale_f32(float* x, long long n, float s, hipStream_t stream);
+// Router of a mixture of experts on float32 logits z [T, E]: scores by sigmoid (softmax over
+// the experts if `softmax`), the `top` largest (lower index on a tie) to idx [T, top], their
+// scores (divided by their sum + norm_eps if `normalize`) to wgt [T, top].
+int hal_moe_route(const float* z, int E, int top, int softmax, int normalize, float norm_eps,
+                  int* idx, float* wgt, int n_tokens, hipStream_t stream);
+// Counting sort of the n (token, choice) pairs by expert (idx [n]); offsets, tile_offsets
+// [E + 1] and sorted [n] as hal_grouped_gemm takes them (tiles of `tile` rows).
+int hal_moe_sort(const int* idx, int n, int E, int tile, int* offsets, int* tile_offsets,
+                 int* sorted, hipStream_t stream);
+// h[t] += sum_j wgt[t, j] * y[t * top + j]  (h [T, d] and y [T * top, d] float32)
+int hal_moe_combine(float* h, const float* y, const float* wgt, int top, int d, int n_tokens,
+                    hipStream_t stream);
 
 // ---- the head-size-specific library (attention_mfma.hip) ---------------------------------
 int hal_attention_mfma_head_dim();

@@ -1,0 +1,299 @@
+// Small kernels around a latent attention and a mixture of experts.  All arithmetic is
+// float32; T is the element type of activations (float or bf16).
+//
+//   * RMSNorm of the float32 stream with one or two weights at once (the two norms of a
+//     block whose mixer and feed-forward read the same rows), x * rstd * w in float32 and
+//     one rounding at the end;
+//   * the step between the down projections of a latent attention and its cache: norms of
+//     the query latent and of the key/value latent, and the key and value rows that the
+//     paged attention kernels take;
+//   * column ranges copied head by head;
+//   * the router of a mixture of experts: sigmoid scores, the largest `top`, their weights;
+//   * a counting sort of the (token, choice) pairs by expert, on the device;
+//   * the weighted sum of the chosen experts' results, added into the stream.
+#include "hal_common.h"
+#include "hal_api.h"
+
+// ---------------------------------------------------------------------------------
+// out1[r] = T(x * rstd * w1), out2[r] = T(x * rstd * w2) with x = h[rows ? rows[r] : r]
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void norm_pair_kernel(const float* __restrict__ h, const int* __restrict__ rows,
+                                 const void* __restrict__ w1, const void* __restrict__ w2, int w_dtype,
+                                 float eps, T* __restrict__ out1, T* __restrict__ out2, int d) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const float* hr = h + (size_t)(rows ? rows[r] : r) * d;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    const float x = hr[i];
+    ss += x * x;
+  }
+  const float total = block_sum(ss, scratch);
+  const float rstd = 1.0f / sqrtf(total / (float)d + eps);
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    const float x = hr[i] * rstd;
+    out1[(size_t)r * d + i] = from_f32<T>(x * load_as_f32(w1, w_dtype, i));
+    if (w2) out2[(size_t)r * d + i] = from_f32<T>(x * load_as_f32(w2, w_dtype, i));
+  }
+}
+
+extern "C" int hal_norm_pair(const float* h, const int* rows, const void* w1, const void* w2,
+                             int w_dtype, float eps, void* out1, void* out2, int dtype, int n_rows,
+                             int d, hipStream_t stream) {
+  HAL_REQUIRE(n_rows >= 0 && d > 0, "hal_norm_pair: bad sizes rows=%d d=%d", n_rows, d);
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_norm_pair: dtype %d", dtype);
+  HAL_REQUIRE((w2 == nullptr) == (out2 == nullptr), "hal_norm_pair: a second weight and a second result come together");
+  if (n_rows == 0) return 0;
+  int threads = ((d + 3) / 4 + 63) / 64 * 64;
+  if (threads > 1024) threads = 1024;
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(norm_pair_kernel<float>, dim3(n_rows), dim3(threads), 0, stream, h, rows, w1, w2,
+                       w_dtype, eps, (float*)out1, (float*)out2, d);
+  else
+    hipLaunchKernelGGL(norm_pair_kernel<bf16_t>, dim3(n_rows), dim3(threads), 0, stream, h, rows, w1,
+                       w2, w_dtype, eps, (bf16_t*)out1, (bf16_t*)out2, d);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------
+// a [T, lda] float32 holds, per token, the query latent (q_rank, from column q_col0; none
+// if q_rank == 0), then at kv_col0 the key/value latent (kv_rank) and the shared rotated key
+// part (rot, not normed).
+//   cq[t]         = T(rmsnorm(query latent) * wq)
+//   k row of t    = [rotated part (not yet rotated) | T(rmsnorm(latent) * wkv) | 0 ...]   (D)
+//   v row of t    = [0 ...                          | the same                 | 0 ...]   (D)
+// in the packed rows `qkv` at columns k_col0 and k_col0 + D.
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void latent_prep_kernel(const float* __restrict__ a, int lda, int q_col0, int q_rank,
+                                   int kv_col0, int kv_rank, int rot, int D, const void* wq,
+                                   const void* wkv, int w_dtype, float eps, T* __restrict__ cq,
+                                   T* __restrict__ qkv, int row_stride, int k_col0) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const float* ar = a + (size_t)t * lda;
+  if (q_rank > 0) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < q_rank; i += blockDim.x) ss += ar[q_col0 + i] * ar[q_col0 + i];
+    const float rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)q_rank + eps);
+    for (int i = threadIdx.x; i < q_rank; i += blockDim.x)
+      cq[(size_t)t * q_rank + i] = from_f32<T>(ar[q_col0 + i] * rstd * load_as_f32(wq, w_dtype, i));
+  }
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) ss += ar[kv_col0 + i] * ar[kv_col0 + i];
+  const float rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)kv_rank + eps);
+  T* k = qkv + (size_t)t * row_stride + k_col0;
+  T* v = k + D;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    float kx = 0.f, vx = 0.f;
+    if (i < rot) {
+      kx = ar[kv_col0 + kv_rank + i];
+    } else if (i < rot + kv_rank) {
+      const int c = i - rot;
+      // rounded once, so that keys and values hold the same number
+      kx = vx = to_f32(from_f32<T>(ar[kv_col0 + c] * rstd * load_as_f32(wkv, w_dtype, c)));
+    }
+    k[i] = from_f32<T>(kx);
+    v[i] = from_f32<T>(vx);
+  }
+}
+
+extern "C" int hal_latent_prep(const float* a, int lda, int q_col0, int q_rank, int kv_col0,
+                               int kv_rank, int rot, int D, const void* wq, const void* wkv,
+                               int w_dtype, float eps, void* cq, void* qkv, int row_stride,
+                               int k_col0, int dtype, int n_tokens, hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && kv_rank > 0 && rot >= 0 && q_rank >= 0 && D >= rot + kv_rank,
+              "hal_latent_prep: bad sizes T=%d q_rank=%d kv_rank=%d rot=%d D=%d", n_tokens, q_rank, kv_rank,
+              rot, D);
+  HAL_REQUIRE(q_col0 >= 0 && kv_col0 >= 0 && q_col0 + q_rank <= lda && kv_col0 + kv_rank + rot <= lda &&
+                  k_col0 >= 0 && k_col0 + 2 * D <= row_stride,
+              "hal_latent_prep: columns outside the rows");
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_latent_prep: dtype %d", dtype);
+  if (n_tokens == 0) return 0;
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(latent_prep_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, a, lda, q_col0,
+                       q_rank, kv_col0, kv_rank, rot, D, wq, wkv, w_dtype, eps, (float*)cq, (float*)qkv,
+                       row_stride, k_col0);
+  else
+    hipLaunchKernelGGL(latent_prep_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream, a, lda, q_col0,
+                       q_rank, kv_col0, kv_rank, rot, D, wq, wkv, w_dtype, eps, (bf16_t*)cq,
+                       (bf16_t*)qkv, row_stride, k_col0);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------
+// y[t, h * ys + y0 + j] = x[t, h * xs + x0 + j] for j < n, and zero for the `n_zero` columns
+// from h * ys + z0 on
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void head_cols_kernel(const T* __restrict__ x, int ldx, int xs, int x0, T* __restrict__ y,
+                                 int ldy, int ys, int y0, int n, int z0, int n_zero, int H) {
+  const int t = blockIdx.x;
+  const int per = n + n_zero;
+  for (int e = threadIdx.x; e < H * per; e += blockDim.x) {
+    const int h = e / per, j = e % per;
+    if (j < n) y[(size_t)t * ldy + h * ys + y0 + j] = x[(size_t)t * ldx + h * xs + x0 + j];
+    else y[(size_t)t * ldy + h * ys + z0 + (j - n)] = from_f32<T>(0.f);
+  }
+}
+
+extern "C" int hal_head_cols(const void* x, int ldx, int xs, int x0, void* y, int ldy, int ys, int y0,
+                             int n, int z0, int n_zero, int H, int dtype, int n_tokens,
+                             hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && H > 0 && n >= 0 && n_zero >= 0, "hal_head_cols: bad sizes");
+  HAL_REQUIRE(x0 >= 0 && x0 + n <= xs && H * xs <= ldx && y0 >= 0 && y0 + n <= ys && z0 >= 0 &&
+                  z0 + n_zero <= ys && H * ys <= ldy,
+              "hal_head_cols: columns outside the rows");
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_head_cols: dtype %d", dtype);
+  if (n_tokens == 0 || n + n_zero == 0) return 0;
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(head_cols_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, (const float*)x, ldx,
+                       xs, x0, (float*)y, ldy, ys, y0, n, z0, n_zero, H);
+  else
+    hipLaunchKernelGGL(head_cols_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream, (const bf16_t*)x,
+                       ldx, xs, x0, (bf16_t*)y, ldy, ys, y0, n, z0, n_zero, H);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------
+// x[i] *= s
+// ---------------------------------------------------------------------------------
+__global__ void scale_f32_kernel(float* __restrict__ x, size_t n, float s) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] *= s;
+}
+
+extern "C" int hal_scale_f32(float* x, long long n, float s, hipStream_t stream) {
+  HAL_REQUIRE(n >= 0, "hal_scale_f32: n=%lld", n);
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(scale_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, (size_t)n, s);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------
+// Router: z [T, E] float32 logits.  score = sigmoid(z) (or, softmax == 1, the softmax over
+// the experts); the `top` largest scores (the lower index wins a tie); weights = the chosen
+// scores, divided by their sum + norm_eps if `normalize`.
+// ---------------------------------------------------------------------------------
+__global__ void moe_route_kernel(const float* __restrict__ z, int E, int top, int softmax,
+                                 int normalize, float norm_eps, int* __restrict__ idx,
+                                 float* __restrict__ wgt, int n_tokens) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n_tokens) return;
+  const float* zr = z + (size_t)t * E;
+  float zmax = -INFINITY, denom = 1.f;
+  if (softmax) {
+    for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, zr[e]);
+    denom = 0.f;
+    for (int e = 0; e < E; ++e) denom += expf(zr[e] - zmax);
+  }
+  int* my_idx = idx + (size_t)t * top;
+  float* my_w = wgt + (size_t)t * top;
+  float sum = 0.f;
+  for (int j = 0; j < top; ++j) {
+    int best = -1;
+    float best_s = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      bool taken = false;
+      for (int i = 0; i < j; ++i) taken |= my_idx[i] == e;
+      if (taken) continue;
+      const float s = softmax ? expf(zr[e] - zmax) / denom : 1.0f / (1.0f + expf(-zr[e]));
+      if (best < 0 || s > best_s) best = e, best_s = s;
+    }
+    my_idx[j] = best;
+    my_w[j] = best_s;
+    sum += best_s;
+  }
+  if (normalize)
+    for (int j = 0; j < top; ++j) my_w[j] = my_w[j] / (sum + norm_eps);
+}
+
+extern "C" int hal_moe_route(const float* z, int E, int top, int softmax, int normalize,
+                             float norm_eps, int* idx, float* wgt, int n_tokens,
+                             hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && E > 0 && top > 0 && top <= E, "hal_moe_route: bad sizes T=%d E=%d top=%d",
+              n_tokens, E, top);
+  if (n_tokens == 0) return 0;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((n_tokens + 63) / 64), dim3(64), 0, stream, z, E, top, softmax,
+                     normalize, norm_eps, idx, wgt, n_tokens);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------
+// Counting sort of the n = T * top pairs by expert, one workgroup.  offsets [E + 1]: where
+// each expert's pairs begin in `sorted`; tile_offsets [E + 1]: the same counted in tiles of
+// `tile` rows, each expert's count rounded up; sorted [n]: pair numbers (token * top +
+// choice), expert by expert.  The order inside an expert is not fixed; nothing that is
+// computed from it depends on it.
+// ---------------------------------------------------------------------------------
+#define MOE_MAX_EXPERTS 1024
+__global__ void __launch_bounds__(1024) moe_sort_kernel(const int* __restrict__ idx, int n, int E, int tile,
+                                                        int* __restrict__ offsets,
+                                                        int* __restrict__ tile_offsets,
+                                                        int* __restrict__ sorted) {
+  __shared__ int count[MOE_MAX_EXPERTS];
+  __shared__ int cursor[MOE_MAX_EXPERTS];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int e = idx[i];
+    if (e >= 0 && e < E) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, tiles = 0;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = at;
+      tile_offsets[e] = tiles;
+      cursor[e] = at;
+      at += count[e];
+      tiles += (count[e] + tile - 1) / tile;
+    }
+    offsets[E] = at;
+    tile_offsets[E] = tiles;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int e = idx[i];
+    if (e >= 0 && e < E) sorted[atomicAdd(&cursor[e], 1)] = i;
+  }
+}
+
+extern "C" int hal_moe_sort(const int* idx, int n, int E, int tile, int* offsets, int* tile_offsets,
+                            int* sorted, hipStream_t stream) {
+  HAL_REQUIRE(n >= 0 && E > 0 && E <= MOE_MAX_EXPERTS && tile > 0, "hal_moe_sort: bad sizes n=%d E=%d", n, E);
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, idx, n, E, tile, offsets,
+                     tile_offsets, sorted);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------
+// h[t, :] += sum_j wgt[t, j] * y[t * top + j, :]   (y float32 [T * top, d])
+// ---------------------------------------------------------------------------------
+__global__ void moe_combine_kernel(float* __restrict__ h, const float* __restrict__ y,
+                                   const float* __restrict__ wgt, int top, int d) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float s = 0.f;
+    for (int j = 0; j < top; ++j) s += wgt[(size_t)t * top + j] * y[((size_t)t * top + j) * d + i];
+    h[(size_t)t * d + i] += s;
+  }
+}
+
+extern "C" int hal_moe_combine(float* h, const float* y, const float* wgt, int top, int d,
+                               int n_tokens, hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && top > 0 && d > 0, "hal_moe_combine: bad sizes");
+  if (n_tokens == 0) return 0;
+  int threads = (d + 63) / 64 * 64;
+  if (threads > 256) threads = 256;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(threads), 0, stream, h, y, wgt, top, d);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}

@@ -43,6 +43,8 @@ CORE_SOURCES = [
     "gemm_f32.hip",
     "gemm_bf16.hip",
     "sampling.hip",
+    "grouped_gemm.hip",
+    "latent_moe.hip",
 ]
 ATTENTION_SOURCES = ["runtime.hip", "attention_mfma.hip"]
 

@@ -107,8 +107,8 @@ def _i32(t: torch.Tensor | None, name: str):
 # --------------------------------------------------------------------------------
 
 
-def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None):
-    """``out[t] = table[ids[t]]`` as float32."""
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None, scale: float = 1.0):
+    """``out[t] = table[ids[t]] * scale`` as float32."""
     lib = library.core_library()
     _dev(ids, table, out)
     _i32(ids, "ids")
@@ -118,7 +118,8 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None =
     _need(out.dtype == torch.float32 and out.shape == (n, d), "embedding: bad output")
     _check(
         lib,
-        lib.hal_embedding(_ptr(ids), _ptr(table), dtype_code(table.dtype), _ptr(out), n, d, vocab, _stream()),
+        lib.hal_embedding_scaled(_ptr(ids), _ptr(table), dtype_code(table.dtype), _ptr(out), n, d, vocab,
+                                 ctypes.c_float(scale), _stream()),
     )
     return out
 
@@ -640,3 +641,160 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
             return out
     y = torch.matmul(x, w.t())
     return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
+
+
+# -- products in groups, and the kernels around a latent attention and a mixture of experts --
+
+GROUP_TILE_ROWS = 64  # rows of a tile of the grouped product (what ``moe_sort`` counts tiles in)
+
+
+def rmsnorm_exact(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+                  rows: torch.Tensor | None = None, second: torch.Tensor | None = None):
+    """RMSNorm of the float32 stream ``h`` (only of ``rows`` if given) as ``x * rstd * w``
+    in float32 with one rounding at the end; with ``second`` (another weight for the same
+    rows) both results come back."""
+    lib = library.core_library()
+    _dev(h, weight, rows, second)
+    _i32(rows, "rows")
+    _need(h.dtype == torch.float32 and h.dim() == 2, "rmsnorm: the stream is float32 [T, d]")
+    d = h.shape[1]
+    _need(weight.shape == (d,) and (second is None or (second.shape == (d,) and second.dtype == weight.dtype)),
+          "rmsnorm: weights of the stream's width and of one element type")
+    n = h.shape[0] if rows is None else rows.numel()
+    out1 = torch.empty((n, d), dtype=out_dtype, device=h.device)
+    out2 = torch.empty((n, d), dtype=out_dtype, device=h.device) if second is not None else None
+    _check(lib, lib.hal_norm_pair(_ptr(h), _ptr(rows), _ptr(weight), _ptr(second), dtype_code(weight.dtype),
+                                  ctypes.c_float(eps), _ptr(out1), _ptr(out2), dtype_code(out_dtype), n, d, _stream()))
+    return out1 if second is None else (out1, out2)
+
+
+def latent_prep(a: torch.Tensor, q_col0: int, q_rank: int, kv_col0: int, kv_rank: int, rot: int, head_dim: int,
+                w_q: torch.Tensor | None, w_kv: torch.Tensor, eps: float, qkv: torch.Tensor, k_col0: int):
+    """From the float32 down projections ``a`` of a latent attention: the normed query
+    latent ``[T, q_rank]`` (returned, of ``qkv``'s element type; None if ``q_rank`` is 0),
+    and in the packed rows ``qkv`` the key row ``[rot | normed latent | 0]`` at column
+    ``k_col0`` and the value row ``[0 | normed latent | 0]`` behind it, ``head_dim`` columns each."""
+    lib = library.core_library()
+    _dev(a, w_q, w_kv, qkv)
+    n = a.shape[0]
+    _need(a.dtype == torch.float32 and a.dim() == 2 and qkv.dim() == 2 and qkv.shape[0] == n, "latent_prep: rows")
+    _need(w_kv.numel() == kv_rank and (q_rank == 0 or (w_q is not None and w_q.numel() == q_rank and w_q.dtype == w_kv.dtype)),
+          "latent_prep: norm weights")
+    _need(q_col0 + q_rank <= a.shape[1] and kv_col0 + kv_rank + rot <= a.shape[1] and head_dim >= rot + kv_rank
+          and k_col0 + 2 * head_dim <= qkv.shape[1], "latent_prep: columns")
+    cq = torch.empty((n, q_rank), dtype=qkv.dtype, device=a.device) if q_rank else None
+    _check(lib, lib.hal_latent_prep(
+        _ptr(a), a.shape[1], q_col0, q_rank, kv_col0, kv_rank, rot, head_dim, _ptr(w_q), _ptr(w_kv),
+        dtype_code(w_kv.dtype), ctypes.c_float(eps), _ptr(cq), _ptr(qkv), qkv.shape[1], k_col0,
+        dtype_code(qkv.dtype), n, _stream()))
+    return cq
+
+
+def head_cols(x: torch.Tensor, x_head: int, x0: int, y: torch.Tensor, y_head: int, y0: int, n: int,
+              n_heads: int, zero_from: int = 0, n_zero: int = 0) -> None:
+    """``y[t, h * y_head + y0 + j] = x[t, h * x_head + x0 + j]`` for ``j < n`` and every head,
+    and zeros in the ``n_zero`` columns from ``h * y_head + zero_from``."""
+    lib = library.core_library()
+    _dev(x, y)
+    _need(x.dim() == 2 and y.dim() == 2 and x.shape[0] == y.shape[0] and x.dtype == y.dtype, "head_cols: rows")
+    _check(lib, lib.hal_head_cols(_ptr(x), x.shape[1], x_head, x0, _ptr(y), y.shape[1], y_head, y0, n,
+                                  zero_from, n_zero, n_heads, dtype_code(x.dtype), x.shape[0], _stream()))
+
+
+def scale_(x: torch.Tensor, s: float) -> torch.Tensor:
+    """``x *= s`` in place (float32)."""
+    lib = library.core_library()
+    _dev(x)
+    _need(x.dtype == torch.float32, "scale_: float32")
+    if s != 1.0:
+        _check(lib, lib.hal_scale_f32(_ptr(x), ctypes.c_longlong(x.numel()), ctypes.c_float(s), _stream()))
+    return x
+
+
+def grouped_gemm(
+    x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, n_rows: int,
+    x_group_cols: int = 0, x_col0: int = 0, y_group_cols: int = 0, y_col0: int = 0,
+    w_up: torch.Tensor | None = None, limit: float = 0.0, alpha: float = 0.0,
+    group_offsets: torch.Tensor | None = None, tile_offsets: torch.Tensor | None = None,
+    row_src: torch.Tensor | None = None, src_div: int = 1, row_dst: torch.Tensor | None = None,
+    gate: torch.Tensor | None = None, add: bool = False, mfma: bool = True,
+) -> torch.Tensor:
+    """``y_g = x_g @ w[g].T`` for every group ``g`` of ``w`` ``[G, N, K]`` in one launch
+    (float32 accumulation).  Heads: every group has all ``n_rows`` rows; group ``g`` reads
+    the ``K`` columns from ``g * x_group_cols + x_col0`` of ``x`` and writes the ``N``
+    columns from ``g * y_group_cols + y_col0`` of ``y``; ``gate`` (float32, row-strided)
+    multiplies the result by ``sigmoid(gate[t, g * y_group_cols + n])``.  Experts:
+    ``group_offsets`` / ``tile_offsets`` (from ``moe_sort``) cut a list of ``n_rows`` rows
+    into the groups' slices; row ``i`` reads ``x[row_src[i] // src_div]`` and writes
+    ``y[row_dst[i]]`` (``i`` without the arrays); with ``w_up`` the result is the clamped
+    gated activation of the two products.  ``add``: added into a float32 ``y``."""
+    lib = library.core_library()
+    _dev(w, w_up, group_offsets, tile_offsets, row_src, row_dst)
+    for t in (x, y, gate):
+        _need(t is None or (t.is_cuda and t.dim() == 2 and t.stride(1) == 1), "grouped_gemm: rows on the GPU")
+    _i32(group_offsets, "group_offsets"), _i32(tile_offsets, "tile_offsets"), _i32(row_src, "row_src"), _i32(row_dst, "row_dst")
+    _need(w.dim() == 3 and w.dtype == x.dtype and (w_up is None or (w_up.shape == w.shape and w_up.dtype == w.dtype)),
+          "grouped_gemm: weights [G, N, K] of the rows' element type")
+    g, n, k = w.shape
+    _need(gate is None or gate.dtype == torch.float32, "grouped_gemm: a float32 gate")
+    _need(not add or y.dtype == torch.float32, "grouped_gemm: only a float32 result is added into")
+    if group_offsets is None:
+        _need(x.shape[0] >= n_rows and y.shape[0] >= n_rows, "grouped_gemm: rows")
+        _need((g - 1) * x_group_cols + x_col0 + k <= x.shape[1] and (g - 1) * y_group_cols + y_col0 + n <= y.shape[1],
+              "grouped_gemm: columns outside the rows")
+        _need(gate is None or (gate.shape[0] >= n_rows and (g - 1) * y_group_cols + n <= gate.shape[1]), "grouped_gemm: gate")
+    else:
+        _need(group_offsets.numel() == g + 1 and tile_offsets is not None and tile_offsets.numel() == g + 1, "grouped_gemm: offsets")
+        _need(x_group_cols == 0 and y_group_cols == 0 and x_col0 + k <= x.shape[1] and y_col0 + n <= y.shape[1], "grouped_gemm: columns")
+        _need(row_src is None or row_src.numel() >= n_rows, "grouped_gemm: row_src")
+        _need(row_dst is None or row_dst.numel() >= n_rows, "grouped_gemm: row_dst")
+        _need(row_src is not None or x.shape[0] >= n_rows, "grouped_gemm: rows of x")
+        _need(row_dst is not None or y.shape[0] >= n_rows, "grouped_gemm: rows of y")
+        _need(gate is None, "grouped_gemm: the gate is for groups that share their rows")
+    _check(lib, lib.hal_grouped_gemm(
+        _ptr(x), x.stride(0), x_group_cols, x_col0, _ptr(w), _ptr(w_up), ctypes.c_longlong(n * k), k,
+        dtype_code(x.dtype), _ptr(y), y.stride(0), y_group_cols, y_col0, dtype_code(y.dtype), 1 if add else 0,
+        n_rows, n, k, g, _ptr(group_offsets), _ptr(tile_offsets), _ptr(row_src), src_div, _ptr(row_dst),
+        _ptr(gate), 0 if gate is None else gate.stride(0), ctypes.c_float(limit), ctypes.c_float(alpha),
+        1 if mfma else 0, _stream()))
+    return y
+
+
+def moe_route(z: torch.Tensor, top: int, softmax: bool = False, normalize: bool = True, norm_eps: float = 0.0):
+    """The ``top`` experts of every token from float32 router logits ``z`` ``[T, E]``: indices
+    ``[T, top]`` int32 and weights ``[T, top]`` float32 (sigmoid scores, or the softmax over
+    the experts; divided by their sum + ``norm_eps`` if ``normalize``)."""
+    lib = library.core_library()
+    _dev(z)
+    _need(z.dtype == torch.float32 and z.dim() == 2, "moe_route: float32 logits [T, E]")
+    t, e = z.shape
+    idx = torch.empty((t, top), dtype=torch.int32, device=z.device)
+    wgt = torch.empty((t, top), dtype=torch.float32, device=z.device)
+    _check(lib, lib.hal_moe_route(_ptr(z), e, top, 1 if softmax else 0, 1 if normalize else 0,
+                                  ctypes.c_float(norm_eps), _ptr(idx), _ptr(wgt), t, _stream()))
+    return idx, wgt
+
+
+def moe_sort(idx: torch.Tensor, n_experts: int):
+    """The (token, choice) pairs of ``idx`` ``[T, top]`` sorted by expert on the device:
+    ``offsets`` and ``tile_offsets`` ``[E + 1]`` and ``sorted`` ``[T * top]`` (pair numbers
+    ``token * top + choice``), as ``grouped_gemm`` takes them."""
+    lib = library.core_library()
+    _dev(idx)
+    _i32(idx, "idx")
+    n = idx.numel()
+    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=idx.device)
+    tile_offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=idx.device)
+    order = torch.empty(max(n, 1), dtype=torch.int32, device=idx.device)
+    _check(lib, lib.hal_moe_sort(_ptr(idx), n, n_experts, GROUP_TILE_ROWS, _ptr(offsets), _ptr(tile_offsets), _ptr(order), _stream()))
+    return offsets, tile_offsets, order
+
+
+def moe_combine(h: torch.Tensor, y: torch.Tensor, wgt: torch.Tensor) -> None:
+    """``h[t] += sum_j wgt[t, j] * y[t * top + j]`` (all float32)."""
+    lib = library.core_library()
+    _dev(h, y, wgt)
+    t, top = wgt.shape
+    _need(h.dtype == y.dtype == wgt.dtype == torch.float32 and h.shape[0] == t and y.shape == (t * top, h.shape[1]),
+          "moe_combine: float32 h [T, d], y [T * top, d], weights [T, top]")
+    _check(lib, lib.hal_moe_combine(_ptr(h), _ptr(y), _ptr(wgt), top, h.shape[1], t, _stream()))

@@ -1,4 +1,4 @@
-from . import attention, block, embedding, feedforward, norm, rope  # noqa: F401
+from . import attention, block, embedding, feedforward, latent_attention, moe, norm, rope  # noqa: F401
 from .base import (
     ARRANGEMENTS,
     EMBEDDINGS,

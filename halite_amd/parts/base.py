@@ -160,6 +160,10 @@ class Mixer(Part):
 
     takes_normed_rows: ClassVar[bool] = False
     folds_next_norm: ClassVar[bool] = False
+    # True: ``forward(..., add_to=h)`` adds the part's result into the float32 stream ``h``
+    # itself (and returns None) instead of returning it; arrangements whose parts read the
+    # same rows of the stream ask for this
+    adds_to_stream: ClassVar[bool] = False
 
     def attention_sizes(self) -> tuple[int, int, int] | None:
         """(query heads, key/value heads, head size) if the mixer has such sizes, for the
@@ -179,6 +183,7 @@ class FeedForward(Part):
     # as for Mixer
     takes_normed_rows: ClassVar[bool] = False
     folds_next_norm: ClassVar[bool] = False
+    adds_to_stream: ClassVar[bool] = False
 
     def forward(self, x: torch.Tensor, ctx: "StepContext") -> torch.Tensor:
         raise NotImplementedError

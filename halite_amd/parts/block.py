@@ -10,7 +10,9 @@ per-request state, which the step function binds to every run of the layer.
 
 from __future__ import annotations
 
+from ..kernels import ops
 from .base import FEED_FORWARDS, MIXERS, NORMS, Arrangement, register_arrangement
+from .norm import RMSNorm
 
 
 @register_arrangement("pre_norm")
@@ -46,3 +48,50 @@ class PreNormBlock(Arrangement):
         if next_norm is not None and self.ff.folds_next_norm:
             return self.ff.forward(x, ctx, then=next_norm)
         return self.ff.forward(x, ctx)
+
+
+@register_arrangement("parallel")
+class ParallelBlock(Arrangement):
+    """``h = h + (mixer(norm_a(h)) + ff(norm_b(h)))``: the mixer and the feed-forward read
+    the same rows of the stream, each through a norm of its own; a layer may leave the
+    feed-forward (and its norm) out.
+
+    Both parts are handed the float32 stream to add their result into (``add_to``), so
+    the sum is float32 and nothing is left pending.  Where both norms are RMSNorms of one
+    eps in the unrounded order, one kernel computes the statistic once and writes both
+    results."""
+
+    graph_safe = True
+    roles = {"mixer_norm": NORMS, "mixer": MIXERS, "ff_norm": NORMS, "ff": FEED_FORWARDS}
+    optional = ("ff_norm", "ff")
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        self.mixer_norm, self.ff_norm, self.ff = parts["mixer_norm"], parts.get("ff_norm"), parts.get("ff")
+        if (self.ff is None) != (self.ff_norm is None):
+            raise ValueError("a parallel block has a feed-forward and its norm, or neither")
+        for name, part in (("mixer", self.mixer), ("ff", self.ff)):
+            if part is not None and not getattr(part, "adds_to_stream", False):
+                raise ValueError(f"a parallel block needs parts that add into the stream; {name} ({type(part).__name__}) does not")
+        a, b = self.mixer_norm, self.ff_norm
+        self._one_pass = (
+            isinstance(a, RMSNorm) and isinstance(b, RMSNorm) and a.p.eps == b.p.eps
+            and not a.p.round_before_weight and not b.p.round_before_weight
+        )
+
+    def forward(self, h, pending, ctx, run):
+        if pending is not None:
+            ops.residual_add(h, pending)
+        if self.ff is None:
+            x = self.mixer_norm.forward(h)
+            self.mixer.forward(x, ctx, run, add_to=h)
+            return None
+        if self._one_pass and self.mixer_norm.weight.dtype == self.ff_norm.weight.dtype:
+            x, y = ops.rmsnorm_exact(h, self.mixer_norm.weight, self.mixer_norm.p.eps, self.mixer_norm.build.dtype,
+                                     second=self.ff_norm.weight)
+        else:
+            x, y = self.mixer_norm.forward(h), self.ff_norm.forward(h)
+        # both results are computed before either is added: both parts read the same stream
+        self.mixer.forward(x, ctx, run, add_to=h)
+        self.ff.forward(y, ctx, add_to=h)
+        return None

@@ -13,12 +13,14 @@ from .base import EMBEDDINGS, HEADS, Embedding, Head, ParamDecl
 class EmbeddingParams(BaseModel):
     vocab_size: StrictInt = Field(gt=0)
     size: StrictInt = Field(gt=0)
+    scale: float = 1.0
+    """Every row is multiplied by this on its way into the stream (in float32)."""
 
 
 @EMBEDDINGS.register("embedding")
 class TokenEmbedding(Embedding):
-    """Row lookup without a multiplier (embedding.py:36-44) into the float32
-    residual stream."""
+    """Row lookup (embedding.py:36-44) into the float32 residual stream, times ``scale``
+    (1 in the reference's models)."""
 
     Params = EmbeddingParams
     graph_safe = True
@@ -27,13 +29,15 @@ class TokenEmbedding(Embedding):
         return {"weight": ParamDecl((self.p.vocab_size, self.p.size))}
 
     def forward(self, tokens):
-        return ops.embedding(tokens, self.weight)
+        return ops.embedding(tokens, self.weight, scale=self.p.scale)
 
 
 class LinearHeadParams(BaseModel):
     vocab_size: StrictInt = Field(gt=0)
     size: StrictInt = Field(gt=0)
     tied: StrictBool = False
+    logit_scale: float = 1.0
+    """The float32 logits are multiplied by this."""
 
 
 @HEADS.register("linear_head")
@@ -61,4 +65,4 @@ class LinearHead(Head):
             self.t_weight = ops.tile_weight(self.weight)
 
     def forward(self, x):
-        return ops.linear(x, self.weight, out_dtype=torch.float32, tiled=self.t_weight)
+        return ops.scale_(ops.linear(x, self.weight, out_dtype=torch.float32, tiled=self.t_weight), self.p.logit_scale)

@@ -1,0 +1,122 @@
+"""A mixture of small gated feed-forward layers with a router, and an optional expert
+that every token uses.
+
+The router's logits are a float32 product; a kernel turns them into the chosen experts
+and their weights, a second one sorts the (token, choice) pairs by expert on the device,
+and two grouped products run all experts at once on the sorted rows: gate and up with the
+activation in the epilogue, then down.  A last kernel adds the weighted results into the
+float32 stream.  Nothing is read back to the host, so a step's launches depend on its
+number of tokens alone.
+"""
+
+from __future__ import annotations
+
+from typing import Literal
+
+import torch
+from pydantic import BaseModel, Field, StrictBool, StrictInt, model_validator
+
+from ..kernels import ops
+from .base import FEED_FORWARDS, FeedForward, ParamDecl
+
+
+class ClampedGate(BaseModel):
+    """``g = min(W_gate x, limit)``, ``u = clamp(W_up x, -limit, limit)``,
+    ``y = g * sigmoid(alpha * g) * (u + 1)``."""
+
+    intermediate_size: StrictInt = Field(gt=0)
+    limit: float = Field(gt=0)
+    alpha: float = 1.702
+
+
+class MoEParams(BaseModel):
+    hidden_size: StrictInt = Field(gt=0)
+    n_experts: StrictInt = Field(gt=0)
+    top_k: StrictInt = Field(gt=0)
+    expert: ClampedGate
+    shared: ClampedGate | None = None
+    score: Literal["sigmoid", "softmax"] = "sigmoid"
+    normalize: StrictBool = True
+    """The chosen scores are divided by their sum (+ ``norm_eps``)."""
+    norm_eps: float = 1e-20
+
+    @model_validator(mode="after")
+    def _check(self):
+        if self.top_k > self.n_experts:
+            raise ValueError(f"top_k {self.top_k} of {self.n_experts} experts")
+        return self
+
+
+@FEED_FORWARDS.register("moe")
+class MixtureOfExperts(FeedForward):
+    Params = MoEParams
+    graph_safe = True
+    adds_to_stream = True
+
+    def param_decls(self):
+        p = self.p
+        d, f = p.hidden_size, p.expert.intermediate_size
+        decls = {"router.weight": ParamDecl((p.n_experts, d))}
+        for e in range(p.n_experts):
+            decls[f"experts.{e}.gate.weight"] = ParamDecl((f, d))
+            decls[f"experts.{e}.up.weight"] = ParamDecl((f, d))
+            decls[f"experts.{e}.down.weight"] = ParamDecl((d, f))
+        if p.shared is not None:
+            fs = p.shared.intermediate_size
+            decls["shared.gate.weight"] = ParamDecl((fs, d))
+            decls["shared.up.weight"] = ParamDecl((fs, d))
+            decls["shared.down.weight"] = ParamDecl((d, fs))
+        return decls
+
+    def allocate(self, dtypes):
+        p = self.p
+        d, f, n, dev = p.hidden_size, p.expert.intermediate_size, p.n_experts, self.build.device
+        kinds = {dt for name, dt in dtypes.items() if name != "router.weight"}
+        if len(kinds) != 1:
+            raise ValueError("the experts' weights are stored with different element types")
+        dt = kinds.pop()
+        # all experts in one tensor per projection: the grouped products index them by expert
+        self.w_gate = torch.empty((n, f, d), dtype=dt, device=dev)
+        self.w_up = torch.empty((n, f, d), dtype=dt, device=dev)
+        self.w_down = torch.empty((n, d, f), dtype=dt, device=dev)
+        self.w_router = torch.empty((n, d), dtype=dtypes["router.weight"], device=dev)
+        out = {"router.weight": self.w_router}
+        for e in range(n):
+            out[f"experts.{e}.gate.weight"] = self.w_gate[e]
+            out[f"experts.{e}.up.weight"] = self.w_up[e]
+            out[f"experts.{e}.down.weight"] = self.w_down[e]
+        if p.shared is not None:
+            fs = p.shared.intermediate_size
+            self.ws_gate = torch.empty((1, fs, d), dtype=dt, device=dev)
+            self.ws_up = torch.empty((1, fs, d), dtype=dt, device=dev)
+            self.ws_down = torch.empty((d, fs), dtype=dt, device=dev)
+            out["shared.gate.weight"], out["shared.up.weight"] = self.ws_gate[0], self.ws_up[0]
+            out["shared.down.weight"] = self.ws_down
+        return out
+
+    def finalize(self):
+        self.t_shared_down = None
+        if (self.p.shared is not None and self.build.tiled_weights and self.ws_down.is_cuda
+                and self.ws_down.dtype == torch.bfloat16 and self.ws_down.shape[1] % 8 == 0):
+            self.t_shared_down = ops.tile_weight(self.ws_down)
+
+    def forward(self, x, ctx, add_to=None):
+        p = self.p
+        n, d = x.shape
+        h = add_to if add_to is not None else torch.zeros((n, d), dtype=torch.float32, device=x.device)
+        z = ops.linear(x, self.w_router, out_dtype=torch.float32)
+        idx, wgt = ops.moe_route(z, p.top_k, softmax=p.score == "softmax", normalize=p.normalize, norm_eps=p.norm_eps)
+        offsets, tiles, order = ops.moe_sort(idx, p.n_experts)
+        pairs = n * p.top_k
+        # rows in the sorted order: row i belongs to pair order[i] = token * top_k + choice
+        act = torch.empty((pairs, p.expert.intermediate_size), dtype=x.dtype, device=x.device)
+        ops.grouped_gemm(x, self.w_gate, act, n_rows=pairs, w_up=self.w_up, limit=p.expert.limit, alpha=p.expert.alpha,
+                         group_offsets=offsets, tile_offsets=tiles, row_src=order, src_div=p.top_k)
+        y = torch.empty((pairs, d), dtype=torch.float32, device=x.device)
+        ops.grouped_gemm(act, self.w_down, y, n_rows=pairs, group_offsets=offsets, tile_offsets=tiles, row_dst=order)
+        if p.shared is not None:
+            acts = torch.empty((n, p.shared.intermediate_size), dtype=x.dtype, device=x.device)
+            ops.grouped_gemm(x, self.ws_gate, acts, n_rows=n, w_up=self.ws_up, limit=p.shared.limit, alpha=p.shared.alpha)
+            ops.residual_add(h, ops.linear(acts, self.ws_down, out_dtype=torch.float32, tiled=self.t_shared_down))
+        ops.moe_combine(h, y, wgt)
+        return None if add_to is not None else h.to(x.dtype)

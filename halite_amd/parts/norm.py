@@ -3,7 +3,7 @@
 from __future__ import annotations
 
 import torch
-from pydantic import BaseModel, Field, StrictInt
+from pydantic import BaseModel, Field, StrictBool, StrictInt
 
 from ..kernels import ops
 from .base import NORMS, Norm, ParamDecl
@@ -12,6 +12,10 @@ from .base import NORMS, Norm, ParamDecl
 class RMSNormParams(BaseModel):
     size: StrictInt = Field(gt=0)
     eps: float = Field(gt=0)
+    round_before_weight: StrictBool = True
+    """True: the normalised value is rounded to the activation type before the weight
+    multiplies it (the reference's order).  False: ``x * rstd * w`` in float32 and one
+    rounding at the end."""
 
 
 @NORMS.register("rmsnorm")
@@ -28,6 +32,10 @@ class RMSNorm(Norm):
         return {"weight": ParamDecl((self.p.size,), init="ones")}
 
     def forward(self, h, delta=None, rows=None):
+        if not self.p.round_before_weight:
+            if delta is not None:
+                ops.residual_add(h, delta)
+            return ops.rmsnorm_exact(h, self.weight, self.p.eps, self.build.dtype, rows=rows)
         if isinstance(delta, ops.NormedRows):
             # the product before has added its result into h and prepared these rows
             if delta.weight is not self.weight or rows is not None:
@@ -36,6 +44,6 @@ class RMSNorm(Norm):
         return ops.rmsnorm(h, self.weight, self.p.eps, self.build.dtype, delta=delta, rows=rows)
 
     def foldable(self, h):
-        if self.build.dtype != torch.bfloat16 or not h.is_cuda:
+        if self.build.dtype != torch.bfloat16 or not h.is_cuda or not self.p.round_before_weight:
             return None
         return ops.NextNorm(h, self.weight, self.p.eps)
