@@ -97,7 +97,9 @@ class Families:
     A call inside another measured call (a product that picks its kernel) counts once."""
 
     GEMM = ("linear", "gemm_bf16_skinny", "gemm_bf16_skinny_norm", "qkv_rope_append", "gemm_f32")
-    ELEMENTWISE = ("rmsnorm", "silu_mul", "rope_append", "embedding", "residual_add")
+    GROUPED = ("grouped_gemm",)
+    ELEMENTWISE = ("rmsnorm", "silu_mul", "rope_append", "embedding", "residual_add", "rmsnorm_exact", "latent_prep",
+                   "head_cols", "scale_", "moe_route", "moe_sort", "moe_combine")
 
     def __init__(self):
         self.spans = []
@@ -131,6 +133,8 @@ class Families:
 
         for name in self.GEMM:
             self._wrap(ops, name, "gemm")
+        for name in self.GROUPED:
+            self._wrap(ops, name, "grouped")
         for name in self.ELEMENTWISE:
             self._wrap(ops, name, "elementwise")
         self._wrap(attention_kernels, "paged_attention", "attention")
@@ -295,6 +299,180 @@ def engine_workload(args) -> dict:
     return record
 
 
+# Layers of the Kavuvik design at two sizes that resemble served models, and the Llama layer
+# that is closest to each: the same width, heads and head size, grouped keys and values, and a
+# feed-forward as wide as the experts that one token uses (the chosen ones and the shared one).
+KAVUVIK_SIZES = {
+    "2048-wide": dict(width=2048, heads=16, dim=128, rot_dim=64, vdim=128, q_rank=768, kv_rank=192,
+                      experts=32, top=4, ff=512, shared_ff=1024, kv_heads=4),
+    "4096-wide": dict(width=4096, heads=32, dim=128, rot_dim=64, vdim=128, q_rank=1536, kv_rank=192,
+                      experts=64, top=6, ff=1024, shared_ff=2048, kv_heads=8),
+}
+COMPARISON_VOCAB = 32000
+
+
+def kavuvik_config(s, n_layers, window):
+    mixer = dict(heads=s["heads"], dim=s["dim"], rot_dim=s["rot_dim"], vdim=s["vdim"], q_rank=s["q_rank"],
+                 kv_rank=s["kv_rank"], scale=(s["dim"] + s["rot_dim"]) ** -0.5, rot=dict(base=500000.0, dims=s["rot_dim"]))
+    if window:
+        mixer["mask"] = dict(size=window)
+    mlp = dict(kind="moe", router=dict(experts=s["experts"], top=s["top"]), expert=dict(ff=s["ff"], limit=7.0),
+               shared=dict(ff=s["shared_ff"], limit=7.0))
+    return dict(architecture="Kavuvik", vocab=COMPARISON_VOCAB, width=s["width"], embedding=dict(scale=1.0),
+                norm=dict(eps=1e-6), logit_scale=1.0, max_positions=8192,
+                layers=[dict(type="latent_attention", mixer=mixer, mlp=mlp) for _ in range(n_layers)])
+
+
+def closest_llama_config(s, n_layers):
+    return dict(LLAMA_3_1_8B, vocab_size=COMPARISON_VOCAB, hidden_size=s["width"], num_hidden_layers=n_layers,
+                num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"], head_dim=s["dim"],
+                intermediate_size=s["top"] * s["ff"] + s["shared_ff"], max_position_embeddings=8192, rope_scaling=None)
+
+
+def kavuvik_work(s, n_layers, tokens, batch=0, kv_tokens=0) -> dict:
+    """Flops of a prompt of ``tokens`` tokens by family (``batch == 0``), or bytes that a decode
+    step of ``batch`` requests with ``kv_tokens`` cached tokens in all has to read, by family."""
+    d, h, D = s["width"], s["heads"], -(-(s["rot_dim"] + s["kv_rank"]) // 16) * 16
+    dense = d * (s["q_rank"] + s["kv_rank"] + s["rot_dim"] + h * s["vdim"]) + s["q_rank"] * h * (s["dim"] + s["rot_dim"]) \
+        + h * s["vdim"] * d + d * s["experts"] + s["shared_ff"] * d
+    heads = h * s["dim"] * s["kv_rank"] + h * s["kv_rank"] * s["vdim"]
+    shared_in = 2 * d * s["shared_ff"]
+    expert = 3 * d * s["ff"]
+    if batch == 0:
+        return {"gemm": 2.0 * tokens * n_layers * dense + 2.0 * COMPARISON_VOCAB * d,
+                "grouped": 2.0 * tokens * n_layers * (heads + shared_in + s["top"] * expert),
+                "attention": 2.0 * tokens * tokens * h * D * n_layers}
+    used = min(s["experts"], batch * s["top"])
+    return {"gemm": 2.0 * (n_layers * dense + COMPARISON_VOCAB * d),
+            "grouped": 2.0 * n_layers * (heads + shared_in + used * expert),
+            "attention": 2.0 * n_layers * kv_tokens * 2 * D}
+
+
+def llama_work(c, n_layers, tokens, batch=0, kv_tokens=0) -> dict:
+    linear = layer_params(c) - 2 * c.hidden_size
+    if batch == 0:
+        return {"gemm": 2.0 * tokens * n_layers * linear + 2.0 * c.vocab_size * c.hidden_size,
+                "attention": 2.0 * tokens * tokens * c.num_attention_heads * c.head_dim * n_layers}
+    return {"gemm": 2.0 * (n_layers * linear + c.vocab_size * c.hidden_size),
+            "attention": 2.0 * n_layers * kv_tokens * 2 * c.num_key_value_heads * c.head_dim}
+
+
+def design_comparison(args) -> dict:
+    """``--workload kavuvik``: prefill and decode throughput of Kavuvik layers at two sizes
+    beside the closest Llama layers, with each family of kernels against its roofline (the
+    products and the attention of a prompt against the bf16 matrix peak, those of a decode
+    step against the memory's bandwidth).  Random weights; a few layers each, named in the record."""
+    import torch
+
+    from halite_amd.config import KavuvikConfig, LlamaConfig, ModelConfig, ServerConfig
+    from halite_amd.engine.batch import Segment
+    from halite_amd.engine.runner import ModelRunner
+
+    n_layers = args.layers or 4
+    prompt, context, batches = args.prefill_tokens, args.context or 2048, (8, 64)
+    gen = torch.Generator().manual_seed(0)
+    peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+
+    def best_ms(fn, reps):
+        times = []
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            times.append(a.elapsed_time(b))
+        return min(times)
+
+    def measure(cfg, work):
+        pool = max(batches) * (context + 128) + prompt + 1024
+        runner = ModelRunner.from_random(
+            cfg, seed=0,
+            server_config=ServerConfig(kv_cache_num_tokens=pool, max_seqs_per_forward=max(batches) + 1,
+                                       max_tokens_per_forward=16384, use_cudagraph=not args.no_graph,
+                                       cudagraph_max_batch_size=max(batches)),
+            model_config=ModelConfig(dtype=args.dtype, context_len=context + 128))
+        vocab = runner.vocab_size
+        out = {"graphs": runner.graphs_allowed, "weights_gb": round(runner.model.param_bytes() / 1e9, 2)}
+
+        def prefill():
+            slot = runner.admit()
+            ids = torch.randint(0, vocab, (prompt,), generator=gen).numpy()
+            runner.step([Segment(slot, 0, ids, [prompt - 1])])
+            runner.free(slot)
+
+        prefill()
+        ms = best_ms(prefill, max(2, args.steps // 16))
+        with Families() as fam:
+            prefill()
+            by = fam.totals_ms()
+        flops = work(prompt)
+        out["prefill"] = {"tokens": prompt, "ms": round(ms, 3), "tok_per_s": round(prompt / ms * 1e3, 1),
+                          "of_peak": round(sum(flops.values()) / (ms * 1e-3) / peak, 4),
+                          "families_ms": {k: round(v, 3) for k, v in by.items()},
+                          "families_of_peak": {k: round(flops[k] / (by[k] * 1e-3) / peak, 4) for k in flops if by.get(k)}}
+        out["decode"] = {}
+        for b in batches:
+            slots = [runner.admit() for _ in range(b)]
+            start = context - args.steps - args.warmup - 8
+            runner.step([Segment(s, 0, torch.randint(0, vocab, (start,), generator=gen).numpy(), []) for s in slots[: b // 2]])
+            runner.step([Segment(s, 0, torch.randint(0, vocab, (start,), generator=gen).numpy(), []) for s in slots[b // 2:]])
+            pos = [start]
+
+            def step():
+                ids = torch.randint(0, vocab, (b,), generator=gen).tolist()
+                runner.step([Segment(s, pos[0], [t], [0]) for s, t in zip(slots, ids)])
+                pos[0] += 1
+
+            for _ in range(args.warmup):
+                step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                step()
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) / args.steps * 1e3
+            graphs, runner.graphs_allowed = runner.graphs_allowed, False
+            with Families() as fam:  # the kernels of one step, launched one by one
+                step()
+                by = fam.totals_ms()
+            runner.graphs_allowed = graphs
+            elt = 2 if args.dtype == "bfloat16" else 4
+            bytes_ = {k: v / 2 * elt for k, v in work(0, b, b * pos[0]).items()}
+            out["decode"][f"batch{b}"] = {
+                "context": pos[0], "ms_per_step": round(ms, 4), "tok_per_s": round(b / ms * 1e3, 1),
+                "of_bandwidth": round(sum(bytes_.values()) / (ms * 1e-3) / HBM_BYTES_PER_S, 4),
+                "families_ms": {k: round(v, 4) for k, v in by.items()},
+                "families_of_bandwidth": {k: round(bytes_[k] / (by[k] * 1e-3) / HBM_BYTES_PER_S, 4) for k in bytes_ if by.get(k)}}
+            for s in slots:
+                runner.free(s)
+        runner.release()
+        return out
+
+    sizes = {}
+    for name, s in KAVUVIK_SIZES.items():
+        kav = KavuvikConfig(**kavuvik_config(s, n_layers, args.window))
+        llama = LlamaConfig(**closest_llama_config(s, n_layers))
+        print(f"[bench] {name}: Kavuvik", file=sys.stderr, flush=True)
+        k = measure(kav, lambda t, b=0, kv=0, s=s: kavuvik_work(s, n_layers, t, b, kv))
+        print(f"[bench] {name}: Llama", file=sys.stderr, flush=True)
+        l = measure(llama, lambda t, b=0, kv=0, c=llama: llama_work(c, n_layers, t, b, kv))
+        sizes[name] = {"shape": s, "kavuvik": k, "llama": l}
+    first = sizes[next(iter(sizes))]["kavuvik"]["decode"]["batch8"]
+    return {
+        "metric": "decode tokens per second of Kavuvik layers (2048-wide, batch 8), beside Llama layers of equal size",
+        "value": first["tok_per_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: seeded uniform-random token ids, random weights N(0, 0.02)",
+        "config": {"model": "Kavuvik and Llama layers", "layers": n_layers, "global_batch": 8, "seq_len": context,
+                   "prefill_tokens": prompt, "window": args.window, "vocab_size": COMPARISON_VOCAB,
+                   "hip_graph": not args.no_graph, "parallelism": "single GPU"},
+        "sizes": sizes,
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -317,8 +495,11 @@ def main() -> int:
                          "by default (scheduling_steps_ahead); 0: read every step's tokens before the next is put together")
     ap.add_argument("--sampling", default="greedy", choices=["greedy", "temperature", "top_p", "top_k", "all"],
                     help="how the decode steps sample (the contract's line is greedy)")
-    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b"],
-                    help="decode8b: the headline line; the others run requests through the scheduler")
+    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b", "kavuvik"],
+                    help="decode8b: the headline line; mixed3b and llama70b run requests through the scheduler; "
+                         "kavuvik: prefill and decode of Kavuvik layers at two sizes beside the closest Llama layers")
+    ap.add_argument("--window", type=int, default=0,
+                    help="kavuvik: the sliding window of its layers (0: none, so that both models attend to the same keys)")
     ap.add_argument("--no-extras", action="store_true",
                     help="leave out what the default line adds beyond the contract's points: contexts of 32,768, "
                          "the 32-bit points and the 3B requests through the scheduler")
@@ -326,6 +507,9 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.workload == "kavuvik":
+        print(json.dumps(design_comparison(args)), flush=True)
+        return 0
     if args.workload != "decode8b":
         print(json.dumps(engine_workload(args)), flush=True)
         return 0
