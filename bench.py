@@ -99,7 +99,7 @@ class Families:
     GEMM = ("linear", "gemm_bf16_skinny", "gemm_bf16_skinny_norm", "qkv_rope_append", "gemm_f32")
     GROUPED = ("grouped_gemm",)
     ELEMENTWISE = ("rmsnorm", "silu_mul", "rope_append", "embedding", "residual_add", "rmsnorm_exact", "latent_prep",
-                   "head_cols", "scale_", "moe_route", "moe_sort", "moe_combine")
+                   "head_cols", "scale_", "moe_route", "moe_sort", "moe_combine", "clamped_gate_mul")
 
     def __init__(self):
         self.spans = []

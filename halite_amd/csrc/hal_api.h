@@ -125,7 +125,7 @@ int hal_sample_spread(const float* logits, int ld, int n_rows, int V, const floa
 // g * y_group_cols + y_col0 of Y's rows (row length ldy, element type y_dtype; y_add: added
 // into a float32 Y).  group_offsets == null: every group has the rows 0 .. M-1.  Otherwise
 // group g has the rows group_offsets[g] .. group_offsets[g + 1] - 1 of a list of M rows in
-// all (tile_offsets: the same counted in tiles of 64 rows, each group rounded up; both
+// all (tile_offsets: the same counted in tiles of 128 rows, each group rounded up; both
 // [G + 1] on the device): row i of the list reads row row_src[i] / src_div of X (i if null)
 // and writes row row_dst[i] of Y (i if null).  W2 != null: two products and the clamped
 // gated activation g = min(x W^T, limit), u = clamp(x W2^T, -limit, limit),
@@ -170,6 +170,11 @@ int hal_moe_sort(const int* idx, int n, int E, int tile, int* offsets, int* tile
 // h[t] += sum_j wgt[t, j] * y[t * top + j]  (h [T, d] and y [T * top, d] float32)
 int hal_moe_combine(float* h, const float* y, const float* wgt, int top, int d, int n_tokens,
                     hipStream_t stream);
+
+// out [T, F] = g * sigmoid(alpha * g) * (u + 1), g = min(gu[t, f], limit), u = clamp(gu[t, F + f],
+// -limit, limit), for rows gu [T, 2F] that hold a gate projection and an up projection.
+int hal_clamped_gate_mul(const void* gu, void* out, int dtype, int n_tokens, int F, float limit,
+                         float alpha, hipStream_t stream);
 
 // ---- the head-size-specific library (attention_mfma.hip) ---------------------------------
 int hal_attention_mfma_head_dim();

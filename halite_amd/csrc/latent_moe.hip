@@ -176,50 +176,80 @@ extern "C" int hal_scale_f32(float* x, long long n, float s, hipStream_t stream)
 }
 
 // ---------------------------------------------------------------------------------
+#define MOE_MAX_EXPERTS 1024
 // Router: z [T, E] float32 logits.  score = sigmoid(z) (or, softmax == 1, the softmax over
 // the experts); the `top` largest scores (the lower index wins a tie); weights = the chosen
 // scores, divided by their sum + norm_eps if `normalize`.
 // ---------------------------------------------------------------------------------
-__global__ void moe_route_kernel(const float* __restrict__ z, int E, int top, int softmax,
-                                 int normalize, float norm_eps, int* __restrict__ idx,
-                                 float* __restrict__ wgt, int n_tokens) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n_tokens) return;
+// One wave a token: lane l holds the scores of the experts l, l + 64, ...; each of the `top`
+// rounds finds the largest score that is left (the lower index on a tie) across the wave.
+#define MOE_ROUTE_PER_LANE (MOE_MAX_EXPERTS / HAL_WAVE)
+__global__ void __launch_bounds__(HAL_WAVE) moe_route_kernel(const float* __restrict__ z, int E, int top, int softmax,
+                                                             int normalize, float norm_eps, int* __restrict__ idx,
+                                                             float* __restrict__ wgt, int n_tokens) {
+  const int t = blockIdx.x, lane = threadIdx.x;
   const float* zr = z + (size_t)t * E;
-  float zmax = -INFINITY, denom = 1.f;
+  float s[MOE_ROUTE_PER_LANE];
+  float zmax = -INFINITY;
+#pragma unroll
+  for (int u = 0; u < MOE_ROUTE_PER_LANE; ++u) {
+    const int e = lane + u * HAL_WAVE;
+    s[u] = e < E ? zr[e] : -INFINITY;
+    zmax = fmaxf(zmax, s[u]);
+  }
   if (softmax) {
-    for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, zr[e]);
-    denom = 0.f;
-    for (int e = 0; e < E; ++e) denom += expf(zr[e] - zmax);
-  }
-  int* my_idx = idx + (size_t)t * top;
-  float* my_w = wgt + (size_t)t * top;
-  float sum = 0.f;
-  for (int j = 0; j < top; ++j) {
-    int best = -1;
-    float best_s = -INFINITY;
-    for (int e = 0; e < E; ++e) {
-      bool taken = false;
-      for (int i = 0; i < j; ++i) taken |= my_idx[i] == e;
-      if (taken) continue;
-      const float s = softmax ? expf(zr[e] - zmax) / denom : 1.0f / (1.0f + expf(-zr[e]));
-      if (best < 0 || s > best_s) best = e, best_s = s;
+    zmax = wave_max(zmax);
+    float part = 0.f;
+#pragma unroll
+    for (int u = 0; u < MOE_ROUTE_PER_LANE; ++u) {
+      s[u] = lane + u * HAL_WAVE < E ? expf(s[u] - zmax) : -INFINITY;
+      part += lane + u * HAL_WAVE < E ? s[u] : 0.f;
     }
-    my_idx[j] = best;
-    my_w[j] = best_s;
-    sum += best_s;
+    const float denom = wave_sum(part);
+#pragma unroll
+    for (int u = 0; u < MOE_ROUTE_PER_LANE; ++u) s[u] = s[u] / denom;
+  } else {
+#pragma unroll
+    for (int u = 0; u < MOE_ROUTE_PER_LANE; ++u)
+      if (lane + u * HAL_WAVE < E) s[u] = 1.0f / (1.0f + expf(-s[u]));
   }
-  if (normalize)
-    for (int j = 0; j < top; ++j) my_w[j] = my_w[j] / (sum + norm_eps);
+  float sum = 0.f;
+  float kept[MOE_ROUTE_PER_LANE];  // lane j % 64 keeps the j-th choice's score in kept[j / 64]
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int best_e = MOE_MAX_EXPERTS;
+#pragma unroll
+    for (int u = 0; u < MOE_ROUTE_PER_LANE; ++u)
+      if (s[u] > best) best = s[u], best_e = lane + u * HAL_WAVE;  // rising index: the lower one stays on a tie
+#pragma unroll
+    for (int off = HAL_WAVE / 2; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, HAL_WAVE);
+      const int oe = __shfl_xor(best_e, off, HAL_WAVE);
+      if (ob > best || (ob == best && oe < best_e)) best = ob, best_e = oe;
+    }
+#pragma unroll
+    for (int u = 0; u < MOE_ROUTE_PER_LANE; ++u)
+      if (lane + u * HAL_WAVE == best_e) s[u] = -INFINITY;  // taken
+    sum += best;
+    if (lane == 0) idx[(size_t)t * top + j] = best_e;
+#pragma unroll
+    for (int u = 0; u < MOE_ROUTE_PER_LANE; ++u)
+      if (u == j / HAL_WAVE && lane == j % HAL_WAVE) kept[u] = best;
+  }
+#pragma unroll
+  for (int u = 0; u < MOE_ROUTE_PER_LANE; ++u) {
+    const int j = lane + u * HAL_WAVE;
+    if (j < top) wgt[(size_t)t * top + j] = normalize ? kept[u] / (sum + norm_eps) : kept[u];
+  }
 }
 
 extern "C" int hal_moe_route(const float* z, int E, int top, int softmax, int normalize,
                              float norm_eps, int* idx, float* wgt, int n_tokens,
                              hipStream_t stream) {
-  HAL_REQUIRE(n_tokens >= 0 && E > 0 && top > 0 && top <= E, "hal_moe_route: bad sizes T=%d E=%d top=%d",
-              n_tokens, E, top);
+  HAL_REQUIRE(n_tokens >= 0 && E > 0 && E <= MOE_MAX_EXPERTS && top > 0 && top <= E,
+              "hal_moe_route: bad sizes T=%d E=%d top=%d", n_tokens, E, top);
   if (n_tokens == 0) return 0;
-  hipLaunchKernelGGL(moe_route_kernel, dim3((n_tokens + 63) / 64), dim3(64), 0, stream, z, E, top, softmax,
+  hipLaunchKernelGGL(moe_route_kernel, dim3(n_tokens), dim3(HAL_WAVE), 0, stream, z, E, top, softmax,
                      normalize, norm_eps, idx, wgt, n_tokens);
   HAL_LAUNCH_CHECK();
   return 0;
@@ -232,7 +262,6 @@ extern "C" int hal_moe_route(const float* z, int E, int top, int softmax, int no
 // choice), expert by expert.  The order inside an expert is not fixed; nothing that is
 // computed from it depends on it.
 // ---------------------------------------------------------------------------------
-#define MOE_MAX_EXPERTS 1024
 __global__ void __launch_bounds__(1024) moe_sort_kernel(const int* __restrict__ idx, int n, int E, int tile,
                                                         int* __restrict__ offsets,
                                                         int* __restrict__ tile_offsets,
@@ -294,6 +323,39 @@ extern "C" int hal_moe_combine(float* h, const float* y, const float* wgt, int t
   int threads = (d + 63) / 64 * 64;
   if (threads > 256) threads = 256;
   hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(threads), 0, stream, h, y, wgt, top, d);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------
+// out[t, f] = g * sigmoid(alpha * g) * (u + 1) with g = min(gu[t, f], limit) and
+// u = clamp(gu[t, F + f], -limit, limit): the activation of a clamped gated feed-forward
+// whose gate and up projections are the two halves of one product's rows.
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void clamped_gate_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int F, float limit,
+                                        float alpha) {
+  const int t = blockIdx.y;
+  const int f = blockIdx.x * blockDim.x + threadIdx.x;
+  if (f >= F) return;
+  const float g = fminf(to_f32(gu[(size_t)t * 2 * F + f]), limit);
+  const float u = fminf(fmaxf(to_f32(gu[(size_t)t * 2 * F + F + f]), -limit), limit);
+  out[(size_t)t * F + f] = from_f32<T>(g / (1.0f + __expf(-alpha * g)) * (u + 1.0f));
+}
+
+extern "C" int hal_clamped_gate_mul(const void* gu, void* out, int dtype, int n_tokens, int F,
+                                    float limit, float alpha, hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && F > 0, "hal_clamped_gate_mul: bad sizes T=%d F=%d", n_tokens, F);
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_clamped_gate_mul: dtype %d", dtype);
+  HAL_REQUIRE(n_tokens <= 65535, "hal_clamped_gate_mul: %d rows", n_tokens);
+  if (n_tokens == 0) return 0;
+  dim3 grid((F + 255) / 256, n_tokens);
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(clamped_gate_mul_kernel<float>, grid, dim3(256), 0, stream, (const float*)gu,
+                       (float*)out, F, limit, alpha);
+  else
+    hipLaunchKernelGGL(clamped_gate_mul_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)gu,
+                       (bf16_t*)out, F, limit, alpha);
   HAL_LAUNCH_CHECK();
   return 0;
 }

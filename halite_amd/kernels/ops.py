@@ -645,7 +645,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
 
 # -- products in groups, and the kernels around a latent attention and a mixture of experts --
 
-GROUP_TILE_ROWS = 64  # rows of a tile of the grouped product (what ``moe_sort`` counts tiles in)
+GROUP_TILE_ROWS = 128  # rows of a tile of the grouped product (what ``moe_sort`` counts tiles in)
 
 
 def rmsnorm_exact(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
@@ -798,3 +798,16 @@ def moe_combine(h: torch.Tensor, y: torch.Tensor, wgt: torch.Tensor) -> None:
     _need(h.dtype == y.dtype == wgt.dtype == torch.float32 and h.shape[0] == t and y.shape == (t * top, h.shape[1]),
           "moe_combine: float32 h [T, d], y [T * top, d], weights [T, top]")
     _check(lib, lib.hal_moe_combine(_ptr(h), _ptr(y), _ptr(wgt), top, h.shape[1], t, _stream()))
+
+
+def clamped_gate_mul(gate_up: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    """``g * sigmoid(alpha * g) * (u + 1)`` with ``g = min(gate, limit)`` and
+    ``u = clamp(up, -limit, limit)`` of rows ``[gate | up]``."""
+    lib = library.core_library()
+    _dev(gate_up)
+    n, two_f = gate_up.shape
+    _need(two_f % 2 == 0, "clamped_gate_mul: odd row length")
+    out = torch.empty((n, two_f // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _check(lib, lib.hal_clamped_gate_mul(_ptr(gate_up), _ptr(out), dtype_code(gate_up.dtype), n, two_f // 2,
+                                         ctypes.c_float(limit), ctypes.c_float(alpha), _stream()))
+    return out

@@ -87,10 +87,10 @@ class MixtureOfExperts(FeedForward):
             out[f"experts.{e}.down.weight"] = self.w_down[e]
         if p.shared is not None:
             fs = p.shared.intermediate_size
-            self.ws_gate = torch.empty((1, fs, d), dtype=dt, device=dev)
-            self.ws_up = torch.empty((1, fs, d), dtype=dt, device=dev)
+            # gate and up in one tensor, gate first: one library product serves both for many rows
+            self.ws_gate_up = torch.empty((2 * fs, d), dtype=dt, device=dev)
             self.ws_down = torch.empty((d, fs), dtype=dt, device=dev)
-            out["shared.gate.weight"], out["shared.up.weight"] = self.ws_gate[0], self.ws_up[0]
+            out["shared.gate.weight"], out["shared.up.weight"] = self.ws_gate_up[:fs], self.ws_gate_up[fs:]
             out["shared.down.weight"] = self.ws_down
         return out
 
@@ -115,8 +115,14 @@ class MixtureOfExperts(FeedForward):
         y = torch.empty((pairs, d), dtype=torch.float32, device=x.device)
         ops.grouped_gemm(act, self.w_down, y, n_rows=pairs, group_offsets=offsets, tile_offsets=tiles, row_dst=order)
         if p.shared is not None:
-            acts = torch.empty((n, p.shared.intermediate_size), dtype=x.dtype, device=x.device)
-            ops.grouped_gemm(x, self.ws_gate, acts, n_rows=n, w_up=self.ws_up, limit=p.shared.limit, alpha=p.shared.alpha)
+            fs = p.shared.intermediate_size
+            if x.dtype == torch.bfloat16 and n <= 16:
+                # few rows: the grouped product of one group, activation in its epilogue
+                acts = torch.empty((n, fs), dtype=x.dtype, device=x.device)
+                ops.grouped_gemm(x, self.ws_gate_up[:fs].view(1, fs, d), acts, n_rows=n, w_up=self.ws_gate_up[fs:].view(1, fs, d),
+                                 limit=p.shared.limit, alpha=p.shared.alpha)
+            else:
+                acts = ops.clamped_gate_mul(ops.linear(x, self.ws_gate_up), p.shared.limit, p.shared.alpha)
             ops.residual_add(h, ops.linear(acts, self.ws_down, out_dtype=torch.float32, tiled=self.t_shared_down))
         ops.moe_combine(h, y, wgt)
         return None if add_to is not None else h.to(x.dtype)

@@ -115,7 +115,7 @@ def test_router(gpu, score, sizes):
     offsets, tiles, order = (a.cpu() for a in ops.moe_sort(idx, e))
     counts = torch.bincount(idx.cpu().flatten().long(), minlength=e)
     assert offsets.tolist() == [0] + torch.cumsum(counts, 0).tolist()
-    assert tiles.tolist() == [0] + torch.cumsum((counts + 63) // 64, 0).tolist()
+    assert tiles.tolist() == [0] + torch.cumsum((counts + 127) // 128, 0).tolist()
     assert sorted(order.tolist()) == list(range(t * top))
     for i in range(e):  # an expert's slice holds the pairs that chose it
         assert all(int(idx.cpu().flatten()[p]) == i for p in order[offsets[i] : offsets[i + 1]].tolist())
