@@ -96,7 +96,7 @@ class Families:
     """HIP events around every call of the kernel wrappers, by family, for one eager step.
     A call inside another measured call (a product that picks its kernel) counts once."""
 
-    GEMM = ("linear", "gemm_bf16_skinny", "gemm_bf16_skinny_norm", "qkv_rope_append", "gemm_f32")
+    GEMM = ("linear", "linear_add", "gemm_bf16_skinny", "gemm_bf16_skinny_norm", "qkv_rope_append", "gemm_f32")
     GROUPED = ("grouped_gemm",)
     ELEMENTWISE = ("rmsnorm", "silu_mul", "rope_append", "embedding", "residual_add", "rmsnorm_exact", "latent_prep",
                    "head_cols", "scale_", "moe_route", "moe_sort", "moe_combine", "clamped_gate_mul")

@@ -167,9 +167,10 @@ int hal_moe_route(const float* z, int E, int top, int softmax, int normalize, fl
 // [E + 1] and sorted [n] as hal_grouped_gemm takes them (tiles of `tile` rows).
 int hal_moe_sort(const int* idx, int n, int E, int tile, int* offsets, int* tile_offsets,
                  int* sorted, hipStream_t stream);
-// h[t] += sum_j wgt[t, j] * y[t * top + j]  (h [T, d] and y [T * top, d] float32)
-int hal_moe_combine(float* h, const float* y, const float* wgt, int top, int d, int n_tokens,
-                    hipStream_t stream);
+// h[t] += sum_j wgt[t, j] * y[t * top + j] (+ extra[t] if given)  (h, extra [T, d] and
+// y [T * top, d] float32)
+int hal_moe_combine(float* h, const float* y, const float* wgt, const float* extra, int top, int d,
+                    int n_tokens, hipStream_t stream);
 
 // out [T, F] = g * sigmoid(alpha * g) * (u + 1), g = min(gu[t, f], limit), u = clamp(gu[t, F + f],
 // -limit, limit), for rows gu [T, 2F] that hold a gate projection and an up projection.

@@ -304,25 +304,26 @@ extern "C" int hal_moe_sort(const int* idx, int n, int E, int tile, int* offsets
 }
 
 // ---------------------------------------------------------------------------------
-// h[t, :] += sum_j wgt[t, j] * y[t * top + j, :]   (y float32 [T * top, d])
+// h[t, :] += sum_j wgt[t, j] * y[t * top + j, :] (+ extra[t, :])   (y float32 [T * top, d])
 // ---------------------------------------------------------------------------------
 __global__ void moe_combine_kernel(float* __restrict__ h, const float* __restrict__ y,
-                                   const float* __restrict__ wgt, int top, int d) {
+                                   const float* __restrict__ wgt, const float* __restrict__ extra, int top,
+                                   int d) {
   const int t = blockIdx.x;
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
-    float s = 0.f;
+    float s = extra ? extra[(size_t)t * d + i] : 0.f;
     for (int j = 0; j < top; ++j) s += wgt[(size_t)t * top + j] * y[((size_t)t * top + j) * d + i];
     h[(size_t)t * d + i] += s;
   }
 }
 
-extern "C" int hal_moe_combine(float* h, const float* y, const float* wgt, int top, int d,
-                               int n_tokens, hipStream_t stream) {
+extern "C" int hal_moe_combine(float* h, const float* y, const float* wgt, const float* extra, int top,
+                               int d, int n_tokens, hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && top > 0 && d > 0, "hal_moe_combine: bad sizes");
   if (n_tokens == 0) return 0;
   int threads = (d + 63) / 64 * 64;
   if (threads > 256) threads = 256;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(threads), 0, stream, h, y, wgt, top, d);
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(threads), 0, stream, h, y, wgt, extra, top, d);
   HAL_LAUNCH_CHECK();
   return 0;
 }
@@ -335,8 +336,8 @@ extern "C" int hal_moe_combine(float* h, const float* y, const float* wgt, int t
 template <typename T>
 __global__ void clamped_gate_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int F, float limit,
                                         float alpha) {
-  const int t = blockIdx.y;
-  const int f = blockIdx.x * blockDim.x + threadIdx.x;
+  const int t = blockIdx.x;
+  const int f = blockIdx.y * blockDim.x + threadIdx.x;
   if (f >= F) return;
   const float g = fminf(to_f32(gu[(size_t)t * 2 * F + f]), limit);
   const float u = fminf(fmaxf(to_f32(gu[(size_t)t * 2 * F + F + f]), -limit), limit);
@@ -347,9 +348,9 @@ extern "C" int hal_clamped_gate_mul(const void* gu, void* out, int dtype, int n_
                                     float limit, float alpha, hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && F > 0, "hal_clamped_gate_mul: bad sizes T=%d F=%d", n_tokens, F);
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_clamped_gate_mul: dtype %d", dtype);
-  HAL_REQUIRE(n_tokens <= 65535, "hal_clamped_gate_mul: %d rows", n_tokens);
+  HAL_REQUIRE((F + 255) / 256 <= 65535, "hal_clamped_gate_mul: %d columns", F);
   if (n_tokens == 0) return 0;
-  dim3 grid((F + 255) / 256, n_tokens);
+  dim3 grid(n_tokens, (F + 255) / 256);
   if (dtype == HAL_F32)
     hipLaunchKernelGGL(clamped_gate_mul_kernel<float>, grid, dim3(256), 0, stream, (const float*)gu,
                        (float*)out, F, limit, alpha);

@@ -584,6 +584,16 @@ def gemm_bf16_skinny_norm(
     return out
 
 
+def linear_add(h: torch.Tensor, x: torch.Tensor, w: torch.Tensor, tiled: torch.Tensor | None = None) -> None:
+    """``h += x @ w.T`` for the float32 stream ``h``: the product is float32 and the sum is
+    made in float32; few bf16 rows do both in one kernel."""
+    m, k = x.shape
+    if (w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and m <= SKINNY_ROWS and tiled is not None and k % 8 == 0):
+        gemm_bf16_skinny(x, tiled, add_to=h, tiled_shape=tuple(w.shape))
+        return
+    residual_add(h, linear(x, w, out_dtype=torch.float32, tiled=tiled))
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None,
            tiled: torch.Tensor | None = None, next_norm: NextNorm | None = None):
     """``x @ w.T`` for a weight ``[out, in]``; ``tiled`` is ``tile_weight(w)`` if the
@@ -790,14 +800,15 @@ def moe_sort(idx: torch.Tensor, n_experts: int):
     return offsets, tile_offsets, order
 
 
-def moe_combine(h: torch.Tensor, y: torch.Tensor, wgt: torch.Tensor) -> None:
-    """``h[t] += sum_j wgt[t, j] * y[t * top + j]`` (all float32)."""
+def moe_combine(h: torch.Tensor, y: torch.Tensor, wgt: torch.Tensor, extra: torch.Tensor | None = None) -> None:
+    """``h[t] += sum_j wgt[t, j] * y[t * top + j] (+ extra[t])`` (all float32)."""
     lib = library.core_library()
-    _dev(h, y, wgt)
+    _dev(h, y, wgt, extra)
     t, top = wgt.shape
+    _need(extra is None or (extra.dtype == torch.float32 and extra.shape == h.shape), "moe_combine: extra like h")
     _need(h.dtype == y.dtype == wgt.dtype == torch.float32 and h.shape[0] == t and y.shape == (t * top, h.shape[1]),
           "moe_combine: float32 h [T, d], y [T * top, d], weights [T, top]")
-    _check(lib, lib.hal_moe_combine(_ptr(h), _ptr(y), _ptr(wgt), top, h.shape[1], t, _stream()))
+    _check(lib, lib.hal_moe_combine(_ptr(h), _ptr(y), _ptr(wgt), _ptr(extra), top, h.shape[1], t, _stream()))
 
 
 def clamped_gate_mul(gate_up: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:

@@ -166,6 +166,6 @@ class LatentAttention(Mixer):
         ops.grouped_gemm(latent, self.w_uv3, heads, n_rows=n, x_group_cols=D, x_col0=p.rope_dim, y_group_cols=p.v_dim,
                          gate=a[:, gate_col0:] if p.output_gate else None)
         if add_to is not None:
-            ops.residual_add(add_to, ops.linear(heads, self.w_out, out_dtype=torch.float32, tiled=self.t_out))
+            ops.linear_add(add_to, heads, self.w_out, tiled=self.t_out)
             return None
         return ops.linear(heads, self.w_out, tiled=self.t_out)

@@ -123,6 +123,7 @@ class MixtureOfExperts(FeedForward):
                                  limit=p.shared.limit, alpha=p.shared.alpha)
             else:
                 acts = ops.clamped_gate_mul(ops.linear(x, self.ws_gate_up), p.shared.limit, p.shared.alpha)
-            ops.residual_add(h, ops.linear(acts, self.ws_down, out_dtype=torch.float32, tiled=self.t_shared_down))
-        ops.moe_combine(h, y, wgt)
+            # the shared expert's result rides along with the weighted sum
+            extra = ops.linear(acts, self.ws_down, out_dtype=torch.float32, tiled=self.t_shared_down)
+        ops.moe_combine(h, y, wgt, extra if p.shared is not None else None)
         return None if add_to is not None else h.to(x.dtype)

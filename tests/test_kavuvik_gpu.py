@@ -358,3 +358,89 @@ def test_groups_and_pages_of_layers_that_differ(folders):
     assert held == [7, math.ceil(100 / 16) - (100 - 33 + 1) // 16, math.ceil(100 / 16) - (100 - 7 + 1) // 16]
     runner.free(slot)
     assert runner.cache.idle()
+
+
+# -- the programs: generation from the command line, the random-weights mode, trace replay -----
+
+
+def test_command_line_and_replay_program(folders, tmp_path):
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder, requests, ref = folders[("A", "float32")]
+    cfg, weights = P.KAV_A, P.random_weights(P.KAV_A, seed=5 + 1)
+    cmd = [sys.executable, os.path.join(root, "bin", "halite_generate"), "--model", folder, "--prompt-ids", "5,17,3,90,9",
+           "sampling.temperature=0", "sampling.max_new_tokens=5", "model.dtype=float32", "server.kv_cache_num_tokens=256"]
+    proc = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    rec = json.loads(proc.stdout.strip().split("\n")[-1])
+    ids = [5, 17, 3, 90, 9]
+    for tok in rec["output_ids"][0]:
+        assert tok == int(torch.argmax(plain_logits(cfg, weights, ids, "float32")[-1]))
+        ids.append(tok)
+    assert len(ids) == 10
+    # the random-weights mode writes a folder of this architecture that the engine then reads
+    cfgfile, out = tmp_path / "c.json", tmp_path / "rand"
+    cfgfile.write_text(json.dumps(P.KAV_C))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "halite_make_random_model"), "--config", str(cfgfile),
+                           "--out", str(out), "--seed", "3", "--dtype", "bfloat16"], capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    # the replay program on that folder: a prompt in two portions and a decoded token, beside a second request
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": [1, 2, 3, 4, 5], "want": [4]}, {"id": "b", "tokens": [7], "want": [0]}], "end": ["b"]},
+        {"step": 1, "entries": [{"id": "a", "tokens": [6, 7], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": [8], "want": [0]}], "end": ["a"]},
+    ]
+    logits = tmp_path / "logits"
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(out), "--dtype", "float32",
+                           "--out", str(logits), "--max-tokens", "128"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                          cwd=root, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.split("\n") if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    from safetensors.torch import load_file
+
+    stored = {k: v.float() for k, v in load_file(str(out / "model.safetensors")).items()}
+    want = P.forward(P.KAV_C, stored, [1, 2, 3, 4, 5, 6, 7, 8]).float()
+    got0 = torch.from_numpy(np.fromfile(logits / "0.f32", dtype="<f4").reshape(2, -1))
+    got2 = torch.from_numpy(np.fromfile(logits / "2.f32", dtype="<f4").reshape(1, -1))
+    scale = max(1.0, float(want.abs().max()))
+    assert float((got0[0] - want[4]).abs().max()) < 5e-5 * scale and float((got2[0] - want[7]).abs().max()) < 5e-5 * scale
+    assert float((got0[1] - P.forward(P.KAV_C, stored, [7]).float()[0]).abs().max()) < 5e-5 * scale
+    assert not (logits / "1.f32").exists()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_through_a_captured_graph(folders, dtype):
+    """Decode steps replayed from a graph give what launches one by one give: every part of
+    the model reads what varies (experts chosen, rows sorted, pages) on the device."""
+    folder, requests, _ = folders[("B", dtype)]
+    prompts = [requests["r0"][:40], requests["r2"][:25], requests["r3"][:70]]
+
+    def run(graphs):
+        server = ServerConfig(kv_cache_num_tokens=512, page_size=16, max_seqs_per_forward=4, use_cudagraph=graphs)
+        runner = ModelRunner.from_pretrained(folder, server, ModelConfig(dtype=dtype))
+        assert runner.graphs_allowed == graphs
+        slots = [runner.admit() for _ in prompts]
+        runner.step([Segment(s, 0, p, []) for s, p in zip(slots, prompts)])
+        rows = []
+        for i in range(12):
+            segs = [Segment(s, len(p) + i, [(7 * i + j) % P.KAV_B["vocab"]], [0]) for j, (s, p) in enumerate(zip(slots, prompts))]
+            rows.append(runner.step(segs).float().cpu().clone())
+            if i == 5:  # eager work of the program between replays
+                extra = runner.admit()
+                runner.step([Segment(extra, 0, [1, 2, 3], [2])])
+                runner.free(extra)
+        for s in slots:
+            runner.free(s)
+        assert runner.cache.idle()
+        return torch.stack(rows), runner.graph_replays
+
+    eager, none = run(False)
+    replayed, count = run(True)
+    assert none == 0 and count >= 10
+    assert float((eager - replayed).abs().max()) <= (1e-5 if dtype == "float32" else 1e-2) * float(eager.abs().max())
