@@ -452,12 +452,14 @@ def design_comparison(args) -> dict:
 
     sizes = {}
     for name, s in KAVUVIK_SIZES.items():
+        if args.sizes and name not in args.sizes.split(","):
+            continue
         kav = KavuvikConfig(**kavuvik_config(s, n_layers, args.window))
         llama = LlamaConfig(**closest_llama_config(s, n_layers))
         print(f"[bench] {name}: Kavuvik", file=sys.stderr, flush=True)
         k = measure(kav, lambda t, b=0, kv=0, s=s: kavuvik_work(s, n_layers, t, b, kv))
         print(f"[bench] {name}: Llama", file=sys.stderr, flush=True)
-        l = measure(llama, lambda t, b=0, kv=0, c=llama: llama_work(c, n_layers, t, b, kv))
+        l = None if args.only_new else measure(llama, lambda t, b=0, kv=0, c=llama: llama_work(c, n_layers, t, b, kv))
         sizes[name] = {"shape": s, "kavuvik": k, "llama": l}
     first = sizes[next(iter(sizes))]["kavuvik"]["decode"]["batch8"]
     return {
@@ -498,6 +500,8 @@ def main() -> int:
     ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b", "kavuvik"],
                     help="decode8b: the headline line; mixed3b and llama70b run requests through the scheduler; "
                          "kavuvik: prefill and decode of Kavuvik layers at two sizes beside the closest Llama layers")
+    ap.add_argument("--sizes", default="", help="kavuvik: only these sizes (names with commas between them)")
+    ap.add_argument("--only-new", action="store_true", help="kavuvik: leave the Llama layers out (for profiles)")
     ap.add_argument("--window", type=int, default=0,
                     help="kavuvik: the sliding window of its layers (0: none, so that both models attend to the same keys)")
     ap.add_argument("--no-extras", action="store_true",

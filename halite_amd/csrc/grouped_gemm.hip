@@ -171,8 +171,13 @@ __device__ __forceinline__ gg_bf16x8 gg_frag(const bf16_t* p, bool valid) {
 // X rows 4 * (l / 16) .. + 3, so a store instruction writes runs of 16 neighbouring columns.
 // K, ldx, ldw and the column offsets are multiples of 8 and the bases 16-byte aligned.
 #define GM_TK 64
+// Where the piece of eight k (q of four in step ks of 32 k) of row r of a 16-row tile lies in
+// the tile-step's KiB: at lane q * 16 + r of the operand, with r's bits turned by q and ks, so
+// that the sixteen lanes of a store (two rows, eight pieces) meet sixteen different banks, and
+// the sixteen lanes of a load (one q, sixteen rows) still read one contiguous quarter KiB.
+__device__ __forceinline__ int gm_slot(int q, int r, int ks) { return q * 16 + (r ^ (q << 2) ^ (ks << 1)); }
 __device__ __forceinline__ int gm_lds_offset(int row, int kc) {  // kc: which piece of eight k
-  return (((row / 16) * (GM_TK / 32) + kc / 4) * 64 + (kc % 4) * 16 + row % 16) * 8;
+  return (((row / 16) * (GM_TK / 32) + kc / 4) * 64 + gm_slot(kc % 4, row % 16, kc / 4)) * 8;
 }
 
 // GATED: the tile's 128 W rows are, for each of the two column halves of the waves, 32 rows of
@@ -244,8 +249,9 @@ __global__ void __launch_bounds__(256, 2) grouped_mfma_kernel(GroupedArgs a) {
         gg_bf16x8 xa[4], wa[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          xa[i] = *(const gg_bf16x8*)&As[(((wm * 4 + i) * (GM_TK / 32) + ks) * 64 + lane) * 8];
-          wa[i] = *(const gg_bf16x8*)&Bs[(((wn * 4 + i) * (GM_TK / 32) + ks) * 64 + lane) * 8];
+          const int slot = gm_slot(lane / 16, lane % 16, ks);
+          xa[i] = *(const gg_bf16x8*)&As[(((wm * 4 + i) * (GM_TK / 32) + ks) * 64 + slot) * 8];
+          wa[i] = *(const gg_bf16x8*)&Bs[(((wn * 4 + i) * (GM_TK / 32) + ks) * 64 + slot) * 8];
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i)
