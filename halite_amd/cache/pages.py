@@ -106,9 +106,12 @@ class CacheGroup:
     def first_needed_page(self, next_position: int) -> int:
         """Logical pages before this one are out of reach of every query at
         ``next_position`` or later."""
-        if self.need.window is None:
-            return 0
-        oldest_key = next_position - self.need.window + 1
+        window, chunk = self.need.window, getattr(self.need, "chunk", None)
+        oldest_key = 0
+        if window is not None:
+            oldest_key = max(oldest_key, next_position - window + 1)
+        if chunk is not None:
+            oldest_key = max(oldest_key, next_position - next_position % chunk)
         return max(0, oldest_key // self.page_size)
 
     # A request's table has no holes behind its first held page: ``released[slot]``
@@ -138,7 +141,7 @@ class CacheGroup:
 
     def release_passed(self, slot: int, next_position: int) -> int:
         """Gives back the pages that no query at ``next_position`` or later reads."""
-        if self.need.window is None:
+        if self._span() is None:
             return 0
         table = self.tables.get(slot)
         if not table:
@@ -176,12 +179,20 @@ class CacheGroup:
     def tokens_held_at_most(self, n_tokens: float) -> float:
         """Cache tokens of this group that ``n_tokens`` tokens of one request take at
         most: all of them, or what a window spans (whole pages, and the one being left)."""
-        if self.need.window is None:
+        span = self._span()
+        if span is None:
             return n_tokens
-        return min(n_tokens, (-(-self.need.window // self.page_size) + 1) * self.page_size)
+        return min(n_tokens, (-(-span // self.page_size) + 1) * self.page_size)
 
     def pages_per_token_span(self, n_tokens: int) -> int:
         """Upper bound of the pages a request of ``n_tokens`` holds at once."""
-        if self.need.window is None:
+        span = self._span()
+        if span is None:
             return -(-n_tokens // self.page_size)
-        return min(-(-n_tokens // self.page_size), -(-self.need.window // self.page_size) + 1)
+        return min(-(-n_tokens // self.page_size), -(-span // self.page_size) + 1)
+
+    def _span(self) -> int | None:
+        """The most keys that a query reaches back over (a window, a chunk, the smaller of
+        both), or None if it reaches back to the request's first token."""
+        spans = [s for s in (self.need.window, getattr(self.need, "chunk", None)) if s is not None]
+        return min(spans) if spans else None

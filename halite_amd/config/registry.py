@@ -43,6 +43,10 @@ class Architecture:
     # pattern of a tensor name in the folder -> parameter path in the model;
     # '#' stands for a layer name (configs/models/llama/checkpoint.py:94-158)
     weight_map: Callable[[BaseModel], dict[str, str]]
+    # Optional: ``(cfg, shape_of) -> cfg`` for a design some of whose sizes are the shapes of
+    # tensors and not keys of the file; ``shape_of(name)`` gives a tensor's shape in the
+    # folder, or None.  ``read_config`` calls it where a folder has tensors.
+    complete_from_tensors: Callable | None = None
 
 
 ARCHITECTURES: dict[str, Architecture] = {}
@@ -95,4 +99,18 @@ def read_config(folder: str) -> tuple[Architecture, BaseModel]:
         raise ConfigError(f"{folder}: no config.json")
     with open(path) as f:
         raw = json.load(f)
-    return parse_config(raw)
+    arch, cfg = parse_config(raw)
+    if arch.complete_from_tensors is not None:
+        from ..weights.safetensors_io import ModelFiles, SafetensorsError
+
+        try:
+            files = ModelFiles(folder)
+        except SafetensorsError:
+            files = None  # (whoever loads the weights reports what is wrong with them)
+        if files is not None:
+            try:
+                names = set(files.names())
+                cfg = arch.complete_from_tensors(cfg, lambda name: tuple(files.shape_of(name)) if name in names else None)
+            finally:
+                files.close()
+    return arch, cfg

@@ -220,7 +220,7 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
                        const int* __restrict__ token_seg, const int* __restrict__ block_table,
                        int bt_stride, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                        float* __restrict__ part, int n_tokens, int H, int K, int D, int page_size,
-                       int n_pages, float scale, int window, int tq, int chunks, int split,
+                       int n_pages, float scale, hal_score_rule rule, int tq, int chunks, int split,
                        int max_pieces, int page_shift, int cw_shift) {
   constexpr int NV = KEYS * R / 16;  // 16-byte vectors of a tile that a thread brings
   constexpr int ROWS_MOST = RW * PLAIN_WAVES;
@@ -251,7 +251,7 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
     int p_max = -1, lo_min = 0x7fffffff;
     for (int t = ta; t < tb; ++t) {
       const int p = positions[t];
-      const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+      const int lo = hal_rule_lo(rule, p);
       p_max = max(p_max, p);
       lo_min = min(lo_min, lo);
     }
@@ -289,7 +289,7 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
       const int r = wave + PLAIN_WAVES * rr;
       const int p = r < n_rows ? positions[ta + r / heads_here] : -1;
       row_p[rr] = p;
-      row_lo[rr] = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+      row_lo[rr] = hal_rule_lo(rule, max(p, 0));
       M[rr] = m[rr] = -INFINITY;
       L[rr] = l[rr] = 0.f;
 #pragma unroll
@@ -355,6 +355,7 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
               dot = dot + other;
             }
             if (valid) s = dot * scale;
+            if (valid && rule.bias) s += hal_rule_bias(rule, h_first + r % heads_here, p - j);
           }
           const float m_new = fmaxf(m[rr], plain_wave_max(s));
           // (a NaN score makes every sum NaN, as it must; m_new is -inf only if no key is valid)
@@ -426,7 +427,7 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
       const bool only_piece = (lo >> piece_shift) == (p >> piece_shift);
       if (r >= n_rows || (split && !(only_piece && blockIdx.z == 0))) continue;
       T* op = out + (size_t)(ta + r / heads_here) * out_row_stride + (size_t)(h_first + r % heads_here) * D;
-      const float inv = 1.0f / L[rr];
+      const float inv = hal_rule_inverse(rule, M[rr], L[rr]);
 #pragma unroll
       for (int c = 0; c < R; ++c) {
         const int d = lane + c * HAL_WAVE;
@@ -442,10 +443,10 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
 template <typename T, int R>
 __global__ void __launch_bounds__(HAL_WAVE)
 attention_plain_merge_kernel(T* __restrict__ out, int out_row_stride, const int* __restrict__ positions,
-                             const float* __restrict__ part, int H, int D, int window, int max_pieces) {
+                             const float* __restrict__ part, int H, int D, hal_score_rule rule, int max_pieces) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int p = positions[t];
-  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int lo = hal_rule_lo(rule, p);
   const int piece_shift = plain_piece_shift(lo, p, max_pieces);
   const int first = lo >> piece_shift, last = p >> piece_shift;
   if (first == last) return;  // written by the piece's own workgroup
@@ -480,7 +481,7 @@ attention_plain_merge_kernel(T* __restrict__ out, int out_row_stride, const int*
     }
   }
   T* op = out + (size_t)t * out_row_stride + (size_t)h * D;
-  const float inv = 1.0f / L;
+  const float inv = hal_rule_inverse(rule, M, L);
 #pragma unroll
   for (int c = 0; c < R; ++c) {
     const int d = lane + c * HAL_WAVE;
@@ -525,7 +526,7 @@ attention_rows_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict__
                       const int* __restrict__ positions, const int* __restrict__ token_seg,
                       const int* __restrict__ block_table, int bt_stride, const T* __restrict__ k_pages,
                       const T* __restrict__ v_pages, int n_tokens, int H, int K, int D, int page_size,
-                      int n_pages, float scale, int window, int tq, int chunks, int page_shift,
+                      int n_pages, float scale, hal_score_rule rule, int tq, int chunks, int page_shift,
                       int cw_shift) {
   constexpr int KEYS = ROWS_KEYS;
   constexpr int NV = KEYS * ((DB + 1) / 2) / 16;
@@ -554,7 +555,7 @@ attention_rows_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict__
     while (tb < t_end && token_seg[tb] == seg) ++tb;
     // (a request's tokens follow each other, so do their positions)
     const int p_first = positions[ta], p_max = positions[tb - 1];
-    const int lo_min = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+    const int lo_min = hal_rule_lo(rule, p_first);
     const int* bt = block_table + (size_t)seg * bt_stride;
     const int n_rows = (tb - ta) * heads_here;
     const int j_begin = lo_min / KEYS * KEYS, j_end = p_max + 1;
@@ -564,13 +565,13 @@ attention_rows_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict__
     const bool have_row = r < n_rows;
     const int token = ta + (have_row ? r / heads_here : 0), head = h_first + (have_row ? r % heads_here : 0);
     const int p = have_row ? positions[token] : -1;
-    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int lo = hal_rule_lo(rule, max(p, 0));
     // what the wave's rows see between them
     const bool wave_has_rows = wave * 32 < n_rows;
     int wave_lo = 0, wave_p = -1;
     if (wave_has_rows) {
       const int p0 = positions[ta + wave * 32 / heads_here];
-      wave_lo = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
+      wave_lo = hal_rule_lo(rule, p0);
       wave_p = positions[ta + min(wave * 32 + 31, n_rows - 1) / heads_here];
     }
     float qreg[DB * 16];
@@ -635,7 +636,7 @@ attention_rows_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict__
       for (int v = 0; v < 16; ++v) {
         const int j = j0 + 8 * (v / 4) + 4 * half + v % 4;
         valid[v] = j >= lo && j <= p;
-        st[v] = valid[v] ? st[v] * scale : -INFINITY;
+        st[v] = valid[v] ? st[v] * scale + (rule.bias ? hal_rule_bias(rule, head, p - j) : 0.f) : -INFINITY;
         mx = fmaxf(mx, st[v]);
       }
       {
@@ -678,7 +679,7 @@ attention_rows_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict__
     }
     if (have_row) {  // element v of a block's 16: dimension 32 b + 8 (v / 4) + 4 half + v % 4
       T* op = out + (size_t)token * out_row_stride + (size_t)head * D;
-      const float inv = 1.0f / l;
+      const float inv = hal_rule_inverse(rule, m, l);
 #pragma unroll
       for (int b = 0; b < DB; ++b)
 #pragma unroll
@@ -750,6 +751,23 @@ extern "C" int hal_attention_simple(const void* q, int q_row_stride, void* out,
                                     int n_tokens, int H, int K, int D, int page_size, int n_pages,
                                     float scale, int window, int max_kv_len, int min_q_len,
                                     hipStream_t stream) {
+  return hal_attention_simple_ruled(q, q_row_stride, out, out_row_stride, dtype, positions, token_seg,
+                                    block_table, bt_stride, k_pages, v_pages, part, n_tokens, H, K, D,
+                                    page_size, n_pages, scale, window, 0, nullptr, 0, 0, max_kv_len,
+                                    min_q_len, stream);
+}
+
+extern "C" int hal_attention_simple_ruled(const void* q, int q_row_stride, void* out,
+                                          int out_row_stride, int dtype, const int* positions,
+                                          const int* token_seg, const int* block_table, int bt_stride,
+                                          const void* k_pages, const void* v_pages, float* part,
+                                          int n_tokens, int H, int K, int D, int page_size, int n_pages,
+                                          float scale, int window, int chunk, const float* bias,
+                                          int bias_len, int sink, int max_kv_len, int min_q_len,
+                                          hipStream_t stream) {
+  HAL_REQUIRE(chunk >= 0 && (bias == nullptr || bias_len > 0),
+              "hal_attention_simple: chunk %d, bias table of %d distances", chunk, bias_len);
+  const hal_score_rule rule = {window, chunk, bias_len, sink ? 1 : 0, bias};
   HAL_REQUIRE(n_tokens >= 0 && H > 0 && K > 0 && D > 0 && page_size > 0 && n_pages > 0,
               "hal_attention_simple: bad sizes T=%d H=%d K=%d D=%d page=%d pages=%d", n_tokens, H,
               K, D, page_size, n_pages);
@@ -782,7 +800,7 @@ extern "C" int hal_attention_simple(const void* q, int q_row_stride, void* out,
   hipLaunchKernelGGL((attention_rows_kernel<T_, DB_>), grid, dim3(PLAIN_THREADS), smem, stream,        \
                      (const T_*)q, q_row_stride, (T_*)out, out_row_stride, positions, token_seg,       \
                      block_table, bt_stride, (const T_*)k_pages, (const T_*)v_pages, n_tokens, H, K, D, \
-                     page_size, n_pages, scale, window, tq, chunks, page_shift, cw_shift)
+                     page_size, n_pages, scale, rule, tq, chunks, page_shift, cw_shift)
 #define ROWS_BY_SIZE(T_)                  \
   do {                                    \
     if (db == 1) ROWS_LAUNCH(T_, 1);      \
@@ -821,11 +839,11 @@ extern "C" int hal_attention_simple(const void* q, int q_row_stride, void* out,
     hipLaunchKernelGGL((attention_plain_kernel<T_, R_, KEYS_, RW_>), grid, dim3(PLAIN_THREADS), smem,     \
                        stream, (const T_*)q, q_row_stride, (T_*)out, out_row_stride, positions,      \
                        token_seg, block_table, bt_stride, (const T_*)k_pages, (const T_*)v_pages,    \
-                       part, n_tokens, H, K, D, page_size, n_pages, scale, window, tq, chunks,       \
+                       part, n_tokens, H, K, D, page_size, n_pages, scale, rule, tq, chunks,         \
                        split, max_pieces, page_shift, cw_shift);                                     \
     if (split)                                                                                      \
       hipLaunchKernelGGL((attention_plain_merge_kernel<T_, R_>), merge_grid, dim3(HAL_WAVE), 0,      \
-                         stream, (T_*)out, out_row_stride, positions, part, H, D, window,            \
+                         stream, (T_*)out, out_row_stride, positions, part, H, D, rule,              \
                          max_pieces);                                                                \
   } while (0)
 #define PLAIN_BY_ROWS(T_, R_)                    \

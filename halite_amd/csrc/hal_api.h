@@ -53,6 +53,18 @@ int hal_attention_simple(const void* q, int q_row_stride, void* out, int out_row
                          int page_size, int n_pages, float scale, int window, int max_kv_len,
                          int min_q_len, hipStream_t stream);
 
+// hal_attention_simple with a rule for the scores: `chunk` > 0: a query sees no key before
+// the start of its own chunk of that many positions; `bias` (or null): float32
+// [H][bias_len], added to the scaled score of the key n tokens back at
+// [head][min(n, bias_len - 1)]; `sink`: one more term of score 0 and no value in the softmax.
+int hal_attention_simple_ruled(const void* q, int q_row_stride, void* out, int out_row_stride,
+                               int dtype, const int* positions, const int* token_seg,
+                               const int* block_table, int bt_stride, const void* k_pages,
+                               const void* v_pages, float* part, int n_tokens, int H, int K, int D,
+                               int page_size, int n_pages, float scale, int window, int chunk,
+                               const float* bias, int bias_len, int sink, int max_kv_len,
+                               int min_q_len, hipStream_t stream);
+
 int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, float* C, int ldc, int M,
                  int N, int K, hipStream_t stream);
 
@@ -176,6 +188,50 @@ int hal_moe_combine(float* h, const float* y, const float* wgt, const float* ext
 // -limit, limit), for rows gu [T, 2F] that hold a gate projection and an up projection.
 int hal_clamped_gate_mul(const void* gu, void* out, int dtype, int n_tokens, int F, float limit,
                          float alpha, hipStream_t stream);
+
+// ---- rows of the stream and of projections (stream_ops.hip) -------------------------------
+// out = T(h), n elements (a multiple of 4)
+int hal_cast_rows(const float* h, void* out, int dtype, long long n, hipStream_t stream);
+// h[r] += a[r] * rsqrt(mean(a[r]^2) + eps) * w (float32 h and a, [n_rows, d]); cast (or
+// null) receives the new rows of h rounded to `dtype`.
+int hal_post_norm_add(float* h, const float* a, const void* w, int w_dtype, float eps, void* cast,
+                      int dtype, int n_rows, int d, hipStream_t stream);
+int hal_relu_squared(const void* x, void* out, int dtype, long long n, hipStream_t stream);
+// y = alpha * y + beta * x
+int hal_scaled_sum_f32(float* y, float alpha, const float* x, float beta, long long n,
+                       hipStream_t stream);
+// From float32 projections q [T, H * dq], k [T, K * dq] and v [T, K * dv] (null: the values
+// are the rows of k as they are; row lengths ldq, ldk, ldv): q and k each divided by the root
+// mean square of their whole row and multiplied by wq, wk; q further by
+// 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) if temp_every > 0; written as
+// packed rows [H heads | K key heads | K value heads] of D entries a head (the rest zero).
+int hal_qk_norm_pack(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
+                     const void* wq, const void* wk, int w_dtype, float eps, const int* positions,
+                     float temp_coef, int temp_every, void* out, int row_stride, int dtype,
+                     int n_tokens, int H, int K, int dq, int dv, int D, hipStream_t stream);
+
+// ---- mixers with a carried state (recurrent.hip) -----------------------------------------
+// y[t, c] = act(bias[c] + sum_j w[c, j] * u[t - taps + 1 + j, c]) over the tokens of each
+// request, the inputs before a step's first token taken from state [slots][taps - 1][C]
+// (float32; zero for a new request).  act: 0 none, 1 silu.  w [C, taps], bias [C] or null.
+int hal_short_conv(const float* u, int ldu, const void* w, const void* bias, int w_dtype, int taps,
+                   const float* state, const int* token_seg, const int* seg_q_start,
+                   const int* token_slot, void* y, int ldy, int y_dtype, int act, int n_tokens,
+                   int C, hipStream_t stream);
+// The state after the step: the last taps - 1 of (the state, then the step's inputs).
+int hal_short_conv_carry(const float* u, int ldu, float* state, int taps, const int* seg_q_start,
+                         const int* seg_q_len, const int* token_slot, int n_segs, int C,
+                         hipStream_t stream);
+// xbc [T, ldx]: x (heads * P), then B and C (groups * N each).  state [slots][heads][N][P].
+// y [T, heads * P] float32 = S_t^T C_t + D x_t.
+int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt_raw, int ld_dt,
+                 const void* dt_bias, const void* a_log, const void* d_skip, int w_dtype,
+                 float* state, const int* seg_q_start, const int* seg_q_len, const int* token_slot,
+                 float* y, int n_segs, int heads, int P, int N, int groups, hipStream_t stream);
+// out = (y * silu(z)) / rms over each of `parts` equal parts of the row * w
+int hal_gated_part_norm(const float* y, const float* z, int ldz, const void* w, int w_dtype,
+                        float eps, void* out, int dtype, int n_tokens, int inner, int parts,
+                        hipStream_t stream);
 
 // ---- the head-size-specific library (attention_mfma.hip) ---------------------------------
 int hal_attention_mfma_head_dim();

@@ -138,6 +138,34 @@ __host__ __device__ __forceinline__ size_t kv_value_offset(bool tiled, int page_
   return (size_t)(slot / 32) * 32 * D + (((d / 16) * 64 + (r / 8) * 16 + d % 16) * 8 + r % 8);
 }
 
+// What an attention kernel does to a score beside scaling it, and which keys a query sees.
+// A query at position p sees the keys lo(p) .. p: no further back than `window` tokens
+// (itself included; 0: no bound) and, with `chunk` > 0, none before the start of its own
+// chunk of that many positions (counted from position 0 of the request).  `bias` (or null):
+// float32 [heads][bias_len], added to the scaled score of a key n tokens back at
+// [head][min(n, bias_len - 1)].  `sink`: the softmax has one more term of score 0 that
+// carries no value (its denominator is 1 + the sum).
+struct hal_score_rule {
+  int window;
+  int chunk;
+  int bias_len;
+  int sink;
+  const float* bias;
+};
+__host__ __device__ __forceinline__ int hal_rule_lo(const hal_score_rule& r, int p) {
+  int lo = 0;
+  if (r.window > 0 && p - r.window + 1 > lo) lo = p - r.window + 1;
+  if (r.chunk > 0 && p - p % r.chunk > lo) lo = p - p % r.chunk;
+  return lo;
+}
+__device__ __forceinline__ float hal_rule_bias(const hal_score_rule& r, int head, int back) {
+  return r.bias[(size_t)head * r.bias_len + (back < r.bias_len ? back : r.bias_len - 1)];
+}
+// 1 / (l + the sink's term) for sums taken relative to the maximum m
+__device__ __forceinline__ float hal_rule_inverse(const hal_score_rule& r, float m, float l) {
+  return 1.0f / (r.sink ? l + expf(-m) : l);
+}
+
 // Sum over a block of up to 1024 threads; every thread gets the result.
 // `scratch` is shared memory for 16 floats.  Safe to call repeatedly with the
 // same scratch.

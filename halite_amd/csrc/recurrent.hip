@@ -1,0 +1,259 @@
+// Kernels of mixers that carry a state of fixed size from token to token: a short causal
+// convolution over time on every channel, and a selective state-space recurrence with a
+// scalar decay per head.  The state lives in float32 rows, one per request slot; a step's
+// tokens come as a flat batch of segments (each the next tokens of one request, in order),
+// described by the step's arrays: for every token its segment and its slot, for every
+// segment where its tokens start and how many there are.
+//
+//   y[t, c] = act(bias[c] + sum_j w[c, j] * u[t - taps + 1 + j, c])   (u = 0 before a request's start)
+//   S_t = exp(-exp(A_log) * dt_t) S_(t-1) + dt_t * B_t x_t^T,  y_t = S_t^T C_t + D x_t,
+//   dt_t = softplus(dt_raw_t + dt_bias)
+//
+// Decays, step sizes, the state and the sums over it are float32 whatever the activations'
+// type is.
+#include "hal_common.h"
+#include "hal_api.h"
+
+#define CONV_MAX_TAPS 16
+
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+
+// ---- the convolution: a thread a (token, channel) ------------------------------------------
+// state [slots][taps - 1][C]: the last taps - 1 inputs of the request before this step
+template <typename TY>
+__global__ void short_conv_kernel(const float* __restrict__ u, int ldu, const void* __restrict__ w,
+                                  const void* __restrict__ bias, int w_dtype, int taps,
+                                  const float* __restrict__ state, const int* __restrict__ token_seg,
+                                  const int* __restrict__ seg_q_start, const int* __restrict__ token_slot,
+                                  TY* __restrict__ y, int ldy, int act, int n_tokens, int C) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int t = blockIdx.x;
+  if (c >= C) return;
+  const int i = t - seg_q_start[token_seg[t]];  // the token's place in its segment
+  const float* st = state + (size_t)token_slot[t] * (taps - 1) * C;
+  float acc = bias ? load_as_f32(bias, w_dtype, c) : 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int back = taps - 1 - j;  // how many tokens before t
+    const float x = back <= i ? u[(size_t)(t - back) * ldu + c] : st[(size_t)(taps - 1 - (back - i)) * C + c];
+    acc = fmaf(load_as_f32(w, w_dtype, (size_t)c * taps + j), x, acc);
+  }
+  if (act == 1) acc = silu_f32(acc);
+  y[(size_t)t * ldy + c] = from_f32<TY>(acc);
+}
+
+extern "C" int hal_short_conv(const float* u, int ldu, const void* w, const void* bias, int w_dtype, int taps,
+                              const float* state, const int* token_seg, const int* seg_q_start,
+                              const int* token_slot, void* y, int ldy, int y_dtype, int act, int n_tokens, int C,
+                              hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && C > 0 && taps >= 1 && taps <= CONV_MAX_TAPS && ldu >= C && ldy >= C,
+              "hal_short_conv: bad sizes T=%d C=%d taps=%d", n_tokens, C, taps);
+  HAL_REQUIRE(y_dtype == HAL_F32 || y_dtype == HAL_BF16, "hal_short_conv: dtype %d", y_dtype);
+  HAL_REQUIRE(act == 0 || act == 1, "hal_short_conv: activation %d", act);
+  HAL_REQUIRE((C + 255) / 256 <= 65535, "hal_short_conv: %d channels exceed the grid limit", C);
+  if (n_tokens == 0) return 0;
+  dim3 grid(n_tokens, (C + 255) / 256);
+  if (y_dtype == HAL_F32)
+    hipLaunchKernelGGL(short_conv_kernel<float>, grid, dim3(256), 0, stream, u, ldu, w, bias, w_dtype, taps, state,
+                       token_seg, seg_q_start, token_slot, (float*)y, ldy, act, n_tokens, C);
+  else
+    hipLaunchKernelGGL(short_conv_kernel<bf16_t>, grid, dim3(256), 0, stream, u, ldu, w, bias, w_dtype, taps, state,
+                       token_seg, seg_q_start, token_slot, (bf16_t*)y, ldy, act, n_tokens, C);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---- what the convolution carries to the next step: a thread a (segment, channel) ---------
+__global__ void short_conv_carry_kernel(const float* __restrict__ u, int ldu, float* __restrict__ state, int taps,
+                                        const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
+                                        const int* __restrict__ token_slot, int C) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int s = blockIdx.y;
+  if (c >= C) return;
+  const int t0 = seg_q_start[s], n = seg_q_len[s];
+  if (n <= 0) return;
+  float* st = state + (size_t)token_slot[t0] * (taps - 1) * C;
+  float keep[CONV_MAX_TAPS];
+  // the last taps - 1 of (what was carried, then the step's inputs)
+#pragma unroll
+  for (int i = 0; i < CONV_MAX_TAPS - 1; ++i) {
+    if (i < taps - 1) {
+      const int at = n + i;  // place in the joined row, whose first taps - 1 are the old ones
+      keep[i] = at < taps - 1 ? st[(size_t)at * C + c] : u[(size_t)(t0 + at - (taps - 1)) * ldu + c];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < CONV_MAX_TAPS - 1; ++i)
+    if (i < taps - 1) st[(size_t)i * C + c] = keep[i];
+}
+
+extern "C" int hal_short_conv_carry(const float* u, int ldu, float* state, int taps, const int* seg_q_start,
+                                    const int* seg_q_len, const int* token_slot, int n_segs, int C,
+                                    hipStream_t stream) {
+  HAL_REQUIRE(n_segs >= 0 && n_segs <= 65535 && C > 0 && taps >= 1 && taps <= CONV_MAX_TAPS && ldu >= C,
+              "hal_short_conv_carry: bad sizes segments=%d C=%d taps=%d", n_segs, C, taps);
+  if (n_segs == 0 || taps == 1) return 0;
+  hipLaunchKernelGGL(short_conv_carry_kernel, dim3((C + 255) / 256, n_segs), dim3(256), 0, stream, u, ldu, state,
+                     taps, seg_q_start, seg_q_len, token_slot, C);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---- the recurrence: a wave takes 64 value channels of one head of one segment and walks
+// the segment's tokens; a lane holds its channel's column of the state (N numbers) in
+// registers, so the sums over the state need no exchange between lanes.  A token's B and C
+// (shared by the lanes) go through LDS, the next token's on their way meanwhile. ------------
+template <typename T, int NREG>
+__global__ void __launch_bounds__(HAL_WAVE)
+ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt_raw, int ld_dt,
+                const void* __restrict__ dt_bias, const void* __restrict__ a_log, const void* __restrict__ d_skip,
+                int w_dtype, float* __restrict__ state, const int* __restrict__ seg_q_start,
+                const int* __restrict__ seg_q_len, const int* __restrict__ token_slot, float* __restrict__ y,
+                int heads, int P, int N, int groups) {
+  __shared__ float bc[2][2 * NREG];
+  const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int p = blockIdx.z * HAL_WAVE + lane;
+  const int t0 = seg_q_start[s], n = seg_q_len[s];
+  if (n <= 0) return;
+  const int inner = heads * P;
+  const int g = h / (heads / groups);
+  const bool live = p < P;
+  float* st = state + (((size_t)token_slot[t0] * heads + h) * N) * P + (live ? p : 0);
+  float S[NREG];
+#pragma unroll
+  for (int i = 0; i < NREG; ++i) S[i] = (live && i < N) ? st[(size_t)i * P] : 0.f;
+  const float rate = expf(load_as_f32(a_log, w_dtype, h));
+  const float bias = load_as_f32(dt_bias, w_dtype, h);
+  const float skip = load_as_f32(d_skip, w_dtype, h);
+  const size_t b_col = (size_t)inner + (size_t)g * N, c_col = (size_t)inner + (size_t)groups * N + (size_t)g * N;
+
+  // a lane brings B[lane], B[lane + 64], .. and the same of C
+  constexpr int PER = (NREG + HAL_WAVE - 1) / HAL_WAVE;
+  float nb[PER], nc[PER];
+  auto ask = [&](int t) {
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int i = lane + u * HAL_WAVE;
+      nb[u] = i < N ? to_f32(xbc[(size_t)t * ldx + b_col + i]) : 0.f;
+      nc[u] = i < N ? to_f32(xbc[(size_t)t * ldx + c_col + i]) : 0.f;
+    }
+  };
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int i = lane + u * HAL_WAVE;
+      if (i < NREG) {
+        bc[buf][i] = nb[u];
+        bc[buf][NREG + i] = nc[u];
+      }
+    }
+  };
+  ask(t0);
+  float x_next = live ? to_f32(xbc[(size_t)t0 * ldx + (size_t)h * P + p]) : 0.f;
+  float dt_next = dt_raw[(size_t)t0 * ld_dt + h];
+  for (int i = 0; i < n; ++i) {
+    const int t = t0 + i, buf = i & 1;
+    put(buf);
+    const float x = x_next, raw = dt_next + bias;
+    if (i + 1 < n) {
+      ask(t + 1);
+      x_next = live ? to_f32(xbc[(size_t)(t + 1) * ldx + (size_t)h * P + p]) : 0.f;
+      dt_next = dt_raw[(size_t)(t + 1) * ld_dt + h];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const float dt = raw > 20.f ? raw : log1pf(expf(raw));
+    const float decay = expf(-rate * dt);
+    const float dtx = dt * x;
+    float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+    for (int k = 0; k < NREG; k += 2) {
+      S[k] = fmaf(decay, S[k], dtx * bc[buf][k]);
+      acc0 = fmaf(S[k], bc[buf][NREG + k], acc0);
+      S[k + 1] = fmaf(decay, S[k + 1], dtx * bc[buf][k + 1]);
+      acc1 = fmaf(S[k + 1], bc[buf][NREG + k + 1], acc1);
+    }
+    if (live) y[(size_t)t * inner + (size_t)h * P + p] = (acc0 + acc1) + skip * x;
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < NREG; ++i)
+      if (i < N) st[(size_t)i * P] = S[i];
+  }
+}
+
+extern "C" int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt_raw, int ld_dt,
+                            const void* dt_bias, const void* a_log, const void* d_skip, int w_dtype, float* state,
+                            const int* seg_q_start, const int* seg_q_len, const int* token_slot, float* y,
+                            int n_segs, int heads, int P, int N, int groups, hipStream_t stream) {
+  HAL_REQUIRE(n_segs >= 0 && heads > 0 && P > 0 && N > 0 && groups > 0 && heads % groups == 0,
+              "hal_ssd_scan: bad sizes segments=%d heads=%d P=%d N=%d groups=%d", n_segs, heads, P, N, groups);
+  HAL_REQUIRE(N <= 256, "hal_ssd_scan: a state of %d numbers a channel exceeds 256", N);
+  HAL_REQUIRE(ldx >= heads * P + 2 * groups * N && ld_dt >= heads, "hal_ssd_scan: rows too short");
+  HAL_REQUIRE(heads <= 65535 && (P + HAL_WAVE - 1) / HAL_WAVE <= 65535, "hal_ssd_scan: grid limit");
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_ssd_scan: dtype %d", dtype);
+  if (n_segs == 0) return 0;
+  dim3 grid(n_segs, heads, (P + HAL_WAVE - 1) / HAL_WAVE);
+#define SCAN_LAUNCH(T_, N_)                                                                                  \
+  hipLaunchKernelGGL((ssd_scan_kernel<T_, N_>), grid, dim3(HAL_WAVE), 0, stream, (const T_*)xbc, ldx, dt_raw, \
+                     ld_dt, dt_bias, a_log, d_skip, w_dtype, state, seg_q_start, seg_q_len, token_slot, y,   \
+                     heads, P, N, groups)
+#define SCAN_BY_STATE(T_)                 \
+  do {                                    \
+    if (N <= 16) SCAN_LAUNCH(T_, 16);     \
+    else if (N <= 32) SCAN_LAUNCH(T_, 32);  \
+    else if (N <= 64) SCAN_LAUNCH(T_, 64);  \
+    else if (N <= 128) SCAN_LAUNCH(T_, 128); \
+    else SCAN_LAUNCH(T_, 256);            \
+  } while (0)
+  if (dtype == HAL_F32)
+    SCAN_BY_STATE(float);
+  else
+    SCAN_BY_STATE(bf16_t);
+#undef SCAN_BY_STATE
+#undef SCAN_LAUNCH
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---- out = norm_g(y * silu(z)) * w: the gate first, then every one of `parts` equal parts of
+// the row divided by its own root mean square; a workgroup a (token, part) -----------------
+template <typename T>
+__global__ void gated_part_norm_kernel(const float* __restrict__ y, const float* __restrict__ z, int ldz,
+                                       const void* __restrict__ w, int w_dtype, float eps, T* __restrict__ out,
+                                       int inner, int parts) {
+  __shared__ float scratch[16];
+  const size_t t = blockIdx.x;
+  const int part = blockIdx.y, n = inner / parts, c0 = part * n;
+  const float* yr = y + t * inner + c0;
+  const float* zr = z + t * ldz + c0;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const float v = yr[i] * silu_f32(zr[i]);
+    ss += v * v;
+  }
+  const float total = block_sum(ss, scratch);
+  const float rstd = 1.0f / sqrtf(total / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const float v = yr[i] * silu_f32(zr[i]);
+    out[t * inner + c0 + i] = from_f32<T>(v * rstd * load_as_f32(w, w_dtype, c0 + i));
+  }
+}
+
+extern "C" int hal_gated_part_norm(const float* y, const float* z, int ldz, const void* w, int w_dtype, float eps,
+                                   void* out, int dtype, int n_tokens, int inner, int parts, hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && inner > 0 && parts > 0 && inner % parts == 0 && parts <= 65535 && ldz >= inner,
+              "hal_gated_part_norm: bad sizes T=%d inner=%d parts=%d", n_tokens, inner, parts);
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_gated_part_norm: dtype %d", dtype);
+  if (n_tokens == 0) return 0;
+  const int n = inner / parts;
+  const int threads = n >= 1024 ? 256 : (n >= 256 ? 128 : 64);
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(gated_part_norm_kernel<float>, dim3(n_tokens, parts), dim3(threads), 0, stream, y, z, ldz, w,
+                       w_dtype, eps, (float*)out, inner, parts);
+  else
+    hipLaunchKernelGGL(gated_part_norm_kernel<bf16_t>, dim3(n_tokens, parts), dim3(threads), 0, stream, y, z, ldz, w,
+                       w_dtype, eps, (bf16_t*)out, inner, parts);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,174 @@
+// Small kernels on rows of the residual stream and of projections.  All arithmetic is
+// float32; T is the element type of activations (float or bf16).
+//
+//   * the stream's rows rounded to the activation type (for a part that reads the stream
+//     itself, without a norm before it);
+//   * a norm on a part's *result*: h += a * rstd(a) * w, in one pass;
+//   * the square of relu;
+//   * y = alpha * y + beta * x on float32 rows (the sum of mixers that run side by side);
+//   * queries and keys normed over the whole projection (all heads at once), the queries
+//     multiplied by a temperature that grows with the logarithm of the position, and
+//     queries, keys and values laid into the packed rows that the kernels which rotate,
+//     append and attend take; the values may be the keys as they were projected.
+#include "hal_common.h"
+#include "hal_api.h"
+
+template <typename T>
+__global__ void cast_rows_kernel(const float* __restrict__ h, T* __restrict__ out, long long n4) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n4) return;
+  float v[4];
+  load4(h + i * 4, v);
+  store4(out + i * 4, v);
+}
+
+extern "C" int hal_cast_rows(const float* h, void* out, int dtype, long long n, hipStream_t stream) {
+  HAL_REQUIRE(n >= 0 && n % 4 == 0, "hal_cast_rows: %lld elements are not a multiple of 4", n);
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_cast_rows: dtype %d", dtype);
+  if (n == 0) return 0;
+  const long long n4 = n / 4;
+  const unsigned blocks = (unsigned)((n4 + 255) / 256);
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(cast_rows_kernel<float>, dim3(blocks), dim3(256), 0, stream, h, (float*)out, n4);
+  else
+    hipLaunchKernelGGL(cast_rows_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, h, (bf16_t*)out, n4);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// h[r] += a[r] * rsqrt(mean(a[r]^2) + eps) * w; cast (or null) receives the new row rounded to T
+template <typename T>
+__global__ void post_norm_add_kernel(float* __restrict__ h, const float* __restrict__ a,
+                                     const void* __restrict__ w, int w_dtype, float eps,
+                                     T* __restrict__ cast, int d) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  const float* ar = a + r * d;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    const float x = ar[i];
+    ss += x * x;
+  }
+  const float total = block_sum(ss, scratch);
+  const float rstd = 1.0f / sqrtf(total / (float)d + eps);
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    const float y = h[r * d + i] + ar[i] * rstd * load_as_f32(w, w_dtype, i);
+    h[r * d + i] = y;
+    if (cast) cast[r * d + i] = from_f32<T>(y);
+  }
+}
+
+extern "C" int hal_post_norm_add(float* h, const float* a, const void* w, int w_dtype, float eps,
+                                 void* cast, int dtype, int n_rows, int d, hipStream_t stream) {
+  HAL_REQUIRE(n_rows >= 0 && d > 0, "hal_post_norm_add: bad sizes rows=%d d=%d", n_rows, d);
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_post_norm_add: dtype %d", dtype);
+  if (n_rows == 0) return 0;
+  const int threads = d >= 1024 ? 256 : (d >= 256 ? 128 : 64);
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(post_norm_add_kernel<float>, dim3(n_rows), dim3(threads), 0, stream, h, a, w, w_dtype, eps,
+                       (float*)cast, d);
+  else
+    hipLaunchKernelGGL(post_norm_add_kernel<bf16_t>, dim3(n_rows), dim3(threads), 0, stream, h, a, w, w_dtype, eps,
+                       (bf16_t*)cast, d);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
+__global__ void relu_squared_kernel(const T* __restrict__ x, T* __restrict__ out, long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float v = fmaxf(to_f32(x[i]), 0.f);
+  out[i] = from_f32<T>(v * v);
+}
+
+extern "C" int hal_relu_squared(const void* x, void* out, int dtype, long long n, hipStream_t stream) {
+  HAL_REQUIRE(n >= 0, "hal_relu_squared: %lld elements", n);
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_relu_squared: dtype %d", dtype);
+  if (n == 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(relu_squared_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)x, (float*)out, n);
+  else
+    hipLaunchKernelGGL(relu_squared_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, (const bf16_t*)x, (bf16_t*)out, n);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+__global__ void scaled_sum_kernel(float* __restrict__ y, float alpha, const float* __restrict__ x, float beta,
+                                  long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) y[i] = __fadd_rn(__fmul_rn(alpha, y[i]), __fmul_rn(beta, x[i]));
+}
+
+extern "C" int hal_scaled_sum_f32(float* y, float alpha, const float* x, float beta, long long n,
+                                  hipStream_t stream) {
+  HAL_REQUIRE(n >= 0, "hal_scaled_sum_f32: %lld elements", n);
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(scaled_sum_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, y, alpha, x, beta, n);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// One workgroup a token.  out row: [H heads of D | K heads of D | K heads of D], a head's
+// first dq (values: dv) entries filled, the rest zero.
+template <typename T>
+__global__ void qk_norm_pack_kernel(const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk,
+                                    const float* __restrict__ v, int ldv, const void* __restrict__ wq,
+                                    const void* __restrict__ wk, int w_dtype, float eps,
+                                    const int* __restrict__ positions, float temp_coef, int temp_every,
+                                    T* __restrict__ out, int row_stride, int H, int K, int dq, int dv, int D) {
+  __shared__ float scratch[16];
+  const size_t t = blockIdx.x;
+  const float* qr = q + t * ldq;
+  const float* kr = k + t * ldk;
+  const float* vr = v ? v + t * ldv : nullptr;
+  const int nq = H * dq, nk = K * dq;
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) sq += qr[i] * qr[i];
+  for (int i = threadIdx.x; i < nk; i += blockDim.x) sk += kr[i] * kr[i];
+  const float tq = block_sum(sq, scratch);
+  const float tk = block_sum(sk, scratch);
+  float rq = 1.0f / sqrtf(tq / (float)nq + eps);
+  const float rk = 1.0f / sqrtf(tk / (float)nk + eps);
+  if (temp_every > 0) {
+    const int p = positions[t];
+    rq *= 1.0f + temp_coef * logf((float)((p + 1) / temp_every + 1));
+  }
+  T* o = out + t * row_stride;
+  for (int e = threadIdx.x; e < H * D; e += blockDim.x) {
+    const int hd = e / D, d = e % D;
+    float x = 0.f;
+    if (d < dq) x = qr[hd * dq + d] * rq * load_as_f32(wq, w_dtype, hd * dq + d);
+    o[e] = from_f32<T>(x);
+  }
+  for (int e = threadIdx.x; e < K * D; e += blockDim.x) {
+    const int hd = e / D, d = e % D;
+    float x = 0.f, y = 0.f;
+    if (d < dq) x = kr[hd * dq + d] * rk * load_as_f32(wk, w_dtype, hd * dq + d);
+    if (d < dv) y = vr ? vr[hd * dv + d] : kr[hd * dq + d];
+    o[H * D + e] = from_f32<T>(x);
+    o[(H + K) * D + e] = from_f32<T>(y);
+  }
+}
+
+extern "C" int hal_qk_norm_pack(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
+                                const void* wq, const void* wk, int w_dtype, float eps, const int* positions,
+                                float temp_coef, int temp_every, void* out, int row_stride, int dtype,
+                                int n_tokens, int H, int K, int dq, int dv, int D, hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && H > 0 && K > 0 && dq > 0 && dv > 0 && D >= dq && D >= dv,
+              "hal_qk_norm_pack: bad sizes T=%d H=%d K=%d dq=%d dv=%d D=%d", n_tokens, H, K, dq, dv, D);
+  HAL_REQUIRE(v != nullptr || dv == dq, "hal_qk_norm_pack: values that are the keys have the keys' size");
+  HAL_REQUIRE(row_stride >= (H + 2 * K) * D, "hal_qk_norm_pack: rows of %d elements are too short", row_stride);
+  HAL_REQUIRE(temp_every == 0 || positions != nullptr, "hal_qk_norm_pack: a temperature needs positions");
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_qk_norm_pack: dtype %d", dtype);
+  if (n_tokens == 0) return 0;
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(qk_norm_pack_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, q, ldq, k, ldk, v, ldv, wq,
+                       wk, w_dtype, eps, positions, temp_coef, temp_every, (float*)out, row_stride, H, K, dq, dv, D);
+  else
+    hipLaunchKernelGGL(qk_norm_pack_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream, q, ldq, k, ldk, v, ldv, wq,
+                       wk, w_dtype, eps, positions, temp_coef, temp_every, (bf16_t*)out, row_stride, H, K, dq, dv, D);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}

@@ -252,9 +252,10 @@ class StepContext:
             )
         return self._groups[group_id]
 
-    def attention(self, q, q_row_stride, kv, group: GroupStep, n_heads, scale, window) -> torch.Tensor:
-        """Attention of every token of the step over its request's cached keys."""
-        return attention_kernels.paged_attention(self, q, q_row_stride, kv, group, n_heads, scale, window)
+    def attention(self, q, q_row_stride, kv, group: GroupStep, n_heads, scale, window, rule=None) -> torch.Tensor:
+        """Attention of every token of the step over its request's cached keys; ``rule``
+        (``kernels.ops.ScoreRule``): a chunked mask, a bias by distance, a sink."""
+        return attention_kernels.paged_attention(self, q, q_row_stride, kv, group, n_heads, scale, window, rule)
 
     def device_plan(self, group_id: int, group_size: int, window: int):
         key = (group_id, group_size, window)

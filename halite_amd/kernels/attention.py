@@ -423,9 +423,10 @@ def upload_plan(plan: AttentionPlan, device):
     return (plan, dev(plan.items), dev(plan.big_items), dev(plan.merges), dev(plan.counts()))
 
 
-def paged_attention(ctx, q, q_row_stride, kv, group, n_heads, scale, window):
+def paged_attention(ctx, q, q_row_stride, kv, group, n_heads, scale, window, rule=None):
     n_pages, n_kv, page_size, head_dim = kv.k.shape
-    if mfma_supported(q.dtype, head_dim, page_size) and q_row_stride % 8 == 0:
+    ruled = rule is not None and not rule.plain()
+    if not ruled and mfma_supported(q.dtype, head_dim, page_size) and q_row_stride % 8 == 0:
         plan_dev = ctx.device_plan(group.group_id, n_heads // n_kv, window)
         if plan_dev is None:
             ctx.plan_attention(group.group_id, n_heads, n_kv, window, head_dim, late=True)
@@ -442,5 +443,5 @@ def paged_attention(ctx, q, q_row_stride, kv, group, n_heads, scale, window):
     fewest = int(ctx.seg_q_len_host.min()) if known else 1
     return ops.attention_simple(
         q, q_row_stride, ctx.positions, ctx.token_seg, group.block_table, kv.k, kv.v, n_heads, scale, window,
-        max_kv_len=most, min_q_len=fewest,
+        max_kv_len=most, min_q_len=fewest, rule=rule,
     )

@@ -45,6 +45,8 @@ CORE_SOURCES = [
     "sampling.hip",
     "grouped_gemm.hip",
     "latent_moe.hip",
+    "stream_ops.hip",
+    "recurrent.hip",
 ]
 ATTENTION_SOURCES = ["runtime.hip", "attention_mfma.hip"]
 

@@ -23,6 +23,23 @@ class KernelError(RuntimeError):
     pass
 
 
+@dataclass(frozen=True)
+class ScoreRule:
+    """What an attention does to its scores beside scaling them, and which keys a query
+    sees beside the causal rule and a window.  ``chunk``: a query sees no key before the
+    start of its own chunk of that many positions (counted from position 0 of the
+    request).  ``bias``: float32 ``[heads, distances]`` on the device, added to the scaled
+    score of the key ``n`` tokens back at ``[head, min(n, distances - 1)]``.  ``sink``: the
+    softmax has one more term of score 0 that carries no value."""
+
+    chunk: int = 0
+    bias: torch.Tensor | None = None
+    sink: bool = False
+
+    def plain(self) -> bool:
+        return self.chunk == 0 and self.bias is None and not self.sink
+
+
 @dataclass
 class NextNorm:
     """What a part's last product is told about the RMSNorm that reads its result: the
@@ -329,6 +346,7 @@ def attention_simple(
     window: int = 0,
     max_kv_len: int | None = None,
     min_q_len: int = 1,
+    rule: ScoreRule | None = None,
 ):
     """Paged attention in float32 arithmetic; ``q`` holds the query heads at the start of
     rows of ``q_row_stride`` elements.  ``max_kv_len``: the most keys that a request of the
@@ -351,13 +369,20 @@ def attention_simple(
                                               ctypes.byref(split), ctypes.byref(rows), ctypes.byref(pieces),
                                               ctypes.byref(floats)))
     part = torch.empty(floats.value, dtype=torch.float32, device=q.device) if floats.value else None
+    rule = rule or ScoreRule()
+    bias = rule.bias
+    if bias is not None:
+        _dev(bias)
+        _need(bias.dtype == torch.float32 and bias.dim() == 2 and bias.shape[0] == n_heads and bias.shape[1] > 0,
+              "attention: the bias is float32 [heads, distances]")
     _check(
         lib,
-        lib.hal_attention_simple(
+        lib.hal_attention_simple_ruled(
             _ptr(q), q_row_stride, _ptr(out), n_heads * head_dim, dtype_code(q.dtype),
             _ptr(positions), _ptr(token_seg), _ptr(block_table), block_table.shape[1],
             _ptr(k_pages), _ptr(v_pages), _ptr(part), n, n_heads, n_kv, head_dim, page_size, n_pages,
-            ctypes.c_float(scale), window, max_kv_len, min_q_len, _stream(),
+            ctypes.c_float(scale), window, rule.chunk, _ptr(bias), 0 if bias is None else bias.shape[1],
+            1 if rule.sink else 0, max_kv_len, min_q_len, _stream(),
         ),
     )
     return out
@@ -821,4 +846,166 @@ def clamped_gate_mul(gate_up: torch.Tensor, limit: float, alpha: float) -> torch
     out = torch.empty((n, two_f // 2), dtype=gate_up.dtype, device=gate_up.device)
     _check(lib, lib.hal_clamped_gate_mul(_ptr(gate_up), _ptr(out), dtype_code(gate_up.dtype), n, two_f // 2,
                                          ctypes.c_float(limit), ctypes.c_float(alpha), _stream()))
+    return out
+
+
+# -- rows of the stream and of projections; mixers with a carried state -----------------------
+
+
+def cast_rows(h: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """The float32 rows ``h`` rounded to ``dtype`` (``h`` itself if that is float32)."""
+    if dtype == torch.float32:
+        return h
+    lib = library.core_library()
+    _dev(h)
+    _need(h.dtype == torch.float32 and h.numel() % 4 == 0, "cast_rows: float32 rows, a multiple of 4 elements")
+    out = torch.empty(h.shape, dtype=dtype, device=h.device)
+    _check(lib, lib.hal_cast_rows(_ptr(h), _ptr(out), dtype_code(dtype), ctypes.c_longlong(h.numel()), _stream()))
+    return out
+
+
+def post_norm_add(h: torch.Tensor, a: torch.Tensor, weight: torch.Tensor, eps: float,
+                  cast_to: torch.dtype | None = None):
+    """``h += a * rsqrt(mean(a^2) + eps) * weight`` row by row in float32 (``h`` and ``a``
+    float32 ``[T, d]``); with ``cast_to`` the new rows rounded to that type come back."""
+    lib = library.core_library()
+    _dev(h, a, weight)
+    _need(h.dtype == torch.float32 and a.dtype == torch.float32 and h.dim() == 2 and a.shape == h.shape,
+          "post_norm_add: float32 rows of one shape")
+    _need(weight.shape == (h.shape[1],), "post_norm_add: weight of the rows' width")
+    cast = None
+    if cast_to is not None and cast_to != torch.float32:
+        cast = torch.empty(h.shape, dtype=cast_to, device=h.device)
+    _check(lib, lib.hal_post_norm_add(_ptr(h), _ptr(a), _ptr(weight), dtype_code(weight.dtype), ctypes.c_float(eps),
+                                      _ptr(cast), dtype_code(cast_to or torch.float32), h.shape[0], h.shape[1], _stream()))
+    return h if cast is None else cast
+
+
+def relu_squared(x: torch.Tensor) -> torch.Tensor:
+    lib = library.core_library()
+    _dev(x)
+    out = torch.empty_like(x)
+    _check(lib, lib.hal_relu_squared(_ptr(x), _ptr(out), dtype_code(x.dtype), ctypes.c_longlong(x.numel()), _stream()))
+    return out
+
+
+def scaled_sum_(y: torch.Tensor, alpha: float, x: torch.Tensor, beta: float) -> torch.Tensor:
+    """``y = alpha * y + beta * x`` in place (float32)."""
+    lib = library.core_library()
+    _dev(y, x)
+    _need(y.dtype == torch.float32 and x.dtype == torch.float32 and x.shape == y.shape, "scaled_sum_: float32 of one shape")
+    _check(lib, lib.hal_scaled_sum_f32(_ptr(y), ctypes.c_float(alpha), _ptr(x), ctypes.c_float(beta),
+                                       ctypes.c_longlong(y.numel()), _stream()))
+    return y
+
+
+def _rows_f32(t: torch.Tensor, cols: int, what: str):
+    _need(t.is_cuda and t.dtype == torch.float32 and t.dim() == 2 and t.stride(1) == 1 and t.shape[1] == cols,
+          f"{what}: float32 rows of {cols} columns on the GPU")
+
+
+def qk_norm_pack(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor | None, w_q: torch.Tensor, w_k: torch.Tensor,
+                 eps: float, n_heads: int, n_kv_heads: int, qk_dim: int, v_dim: int, head_dim: int,
+                 out_dtype: torch.dtype, positions: torch.Tensor | None = None, temp_coef: float = 0.0,
+                 temp_every: int = 0) -> torch.Tensor:
+    """From float32 projections (row-strided views allowed): ``q`` and ``k`` each divided by
+    the root mean square of their whole row (all heads at once) and multiplied by their
+    weights, ``q`` further by ``1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)`` at
+    position ``p`` if ``temp_every`` > 0; the packed rows ``[q heads | k heads | v heads]``
+    of ``head_dim`` entries a head (zero beyond ``qk_dim`` / ``v_dim``) come back.  ``v``
+    None: the values are the keys as they were projected."""
+    lib = library.core_library()
+    n = q.shape[0]
+    _rows_f32(q, n_heads * qk_dim, "qk_norm_pack q"), _rows_f32(k, n_kv_heads * qk_dim, "qk_norm_pack k")
+    if v is not None:
+        _rows_f32(v, n_kv_heads * v_dim, "qk_norm_pack v")
+    _dev(w_q, w_k, positions)
+    _i32(positions, "positions")
+    _need(w_q.numel() == n_heads * qk_dim and w_k.numel() == n_kv_heads * qk_dim and w_q.dtype == w_k.dtype,
+          "qk_norm_pack: norm weights")
+    _need(head_dim >= max(qk_dim, v_dim) and (v is not None or v_dim == qk_dim), "qk_norm_pack: head sizes")
+    _need(temp_every == 0 or (positions is not None and positions.numel() == n), "qk_norm_pack: positions")
+    out = torch.empty((n, (n_heads + 2 * n_kv_heads) * head_dim), dtype=out_dtype, device=q.device)
+    _check(lib, lib.hal_qk_norm_pack(
+        _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), 0 if v is None else v.stride(0), _ptr(w_q), _ptr(w_k),
+        dtype_code(w_q.dtype), ctypes.c_float(eps), _ptr(positions), ctypes.c_float(temp_coef), temp_every,
+        _ptr(out), out.shape[1], dtype_code(out_dtype), n, n_heads, n_kv_heads, qk_dim, v_dim, head_dim, _stream()))
+    return out
+
+
+def short_conv(u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, state: torch.Tensor,
+               token_seg: torch.Tensor, seg_q_start: torch.Tensor, token_slot: torch.Tensor,
+               out_dtype: torch.dtype, silu: bool = False) -> torch.Tensor:
+    """The causal convolution over time ``y[t, c] = act(bias[c] + sum_j weight[c, j] *
+    u[t - taps + 1 + j, c])`` on the step's flat batch: ``u`` float32 ``[T, C]`` (a
+    row-strided view is allowed), ``state`` float32 ``[slots, taps - 1, C]`` the inputs of
+    every request before this step (zeros for a new one; not changed here)."""
+    lib = library.core_library()
+    c, taps = weight.shape
+    _rows_f32(u, c, "short_conv")
+    _dev(weight, bias, state, token_seg, seg_q_start, token_slot)
+    _i32(token_seg, "token_seg"), _i32(seg_q_start, "seg_q_start"), _i32(token_slot, "token_slot")
+    n = u.shape[0]
+    _need(state.dtype == torch.float32 and state.dim() == 3 and state.shape[1:] == (taps - 1, c), "short_conv: state rows")
+    _need(bias is None or (bias.shape == (c,) and bias.dtype == weight.dtype), "short_conv: bias")
+    _need(token_seg.numel() == n and token_slot.numel() == n, "short_conv: one segment and slot a token")
+    y = torch.empty((n, c), dtype=out_dtype, device=u.device)
+    _check(lib, lib.hal_short_conv(
+        _ptr(u), u.stride(0), _ptr(weight), _ptr(bias), dtype_code(weight.dtype), taps, _ptr(state), _ptr(token_seg),
+        _ptr(seg_q_start), _ptr(token_slot), _ptr(y), c, dtype_code(out_dtype), 1 if silu else 0, n, c, _stream()))
+    return y
+
+
+def short_conv_carry(u: torch.Tensor, state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
+                     token_slot: torch.Tensor) -> None:
+    """After ``short_conv``: every request's state becomes the last ``taps - 1`` of (its
+    state, then its inputs of this step)."""
+    lib = library.core_library()
+    c = state.shape[2]
+    _rows_f32(u, c, "short_conv_carry")
+    _dev(state, seg_q_start, seg_q_len, token_slot)
+    _need(state.dtype == torch.float32 and state.dim() == 3, "short_conv_carry: state rows")
+    _need(seg_q_start.numel() == seg_q_len.numel(), "short_conv_carry: segment arrays")
+    _check(lib, lib.hal_short_conv_carry(_ptr(u), u.stride(0), _ptr(state), state.shape[1] + 1, _ptr(seg_q_start),
+                                         _ptr(seg_q_len), _ptr(token_slot), seg_q_start.numel(), c, _stream()))
+
+
+def ssd_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor,
+             d_skip: torch.Tensor, state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
+             token_slot: torch.Tensor, groups: int) -> torch.Tensor:
+    """The state-space recurrence over every request's tokens of the step.  ``xbc``
+    ``[T, heads * P + 2 * groups * N]``: x, then B and C; ``dt_raw`` float32 ``[T, heads]``
+    (a row-strided view is allowed); ``state`` float32 ``[slots, heads, N, P]``, read and
+    left as the step's last state.  Returns float32 ``[T, heads * P]``."""
+    lib = library.core_library()
+    _dev(xbc, dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, token_slot)
+    _, heads, n_state, p = state.shape
+    n = xbc.shape[0]
+    _need(state.dtype == torch.float32 and xbc.dim() == 2 and xbc.shape[1] == heads * p + 2 * groups * n_state,
+          "ssd_scan: rows of x, B and C")
+    _need(dt_raw.is_cuda and dt_raw.dtype == torch.float32 and dt_raw.shape == (n, heads) and dt_raw.stride(1) == 1,
+          "ssd_scan: float32 step sizes [T, heads]")
+    _need(dt_bias.numel() == heads and a_log.numel() == heads and d_skip.numel() == heads
+          and dt_bias.dtype == a_log.dtype == d_skip.dtype, "ssd_scan: one bias, rate and skip a head, of one type")
+    y = torch.empty((n, heads * p), dtype=torch.float32, device=xbc.device)
+    _check(lib, lib.hal_ssd_scan(
+        _ptr(xbc), xbc.shape[1], dtype_code(xbc.dtype), _ptr(dt_raw), dt_raw.stride(0), _ptr(dt_bias), _ptr(a_log),
+        _ptr(d_skip), dtype_code(a_log.dtype), _ptr(state), _ptr(seg_q_start), _ptr(seg_q_len), _ptr(token_slot),
+        _ptr(y), seg_q_start.numel(), heads, p, n_state, groups, _stream()))
+    return y
+
+
+def gated_part_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float, parts: int,
+                    out_dtype: torch.dtype) -> torch.Tensor:
+    """``(y * silu(z))`` with every one of ``parts`` equal parts of a row divided by its
+    own root mean square, times ``weight`` (``y`` float32 ``[T, n]``, ``z`` float32, a
+    row-strided view is allowed)."""
+    lib = library.core_library()
+    _dev(y, weight)
+    n, inner = y.shape
+    _rows_f32(z, inner, "gated_part_norm z")
+    _need(y.dtype == torch.float32 and weight.numel() == inner and inner % parts == 0, "gated_part_norm: sizes")
+    out = torch.empty((n, inner), dtype=out_dtype, device=y.device)
+    _check(lib, lib.hal_gated_part_norm(_ptr(y), _ptr(z), z.stride(0), _ptr(weight), dtype_code(weight.dtype),
+                                        ctypes.c_float(eps), _ptr(out), dtype_code(out_dtype), n, inner, parts, _stream()))
     return out

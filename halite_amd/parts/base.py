@@ -42,7 +42,8 @@ class PagedNeed:
 
     * ``window`` (an attribute; ``None``: every token's page is kept while the request lives;
       else the tokens a query looks back, itself included, so that pages are given back once
-      every later query has passed them);
+      every later query has passed them), and ``chunk`` (likewise; else queries see keys of
+      their own chunk of that many positions only);
     * ``page_tensors(page_size)``: name -> shape of one page, the tensors a run keeps per page
       number, all of the cache's element type;
     * ``bind(group_id, tensors, page_size, dtype)``: what the run's mixer finds in ``run.kv``,
@@ -50,6 +51,7 @@ class PagedNeed:
     """
 
     window: int | None = None
+    chunk: int | None = None
 
     def page_tensors(self, page_size: int) -> dict[str, tuple[int, ...]]:
         raise NotImplementedError
@@ -67,6 +69,12 @@ class PagedKVNeed(PagedNeed):
     n_kv_heads: int
     head_dim: int
     window: int | None = None
+    # a query sees no key before the start of its own chunk of this many positions: pages
+    # that lie wholly before the chunk of the request's next token are given back
+    chunk: int | None = None
+    # True: the pages are kept row by row whatever the sizes (for a reader other than the
+    # matrix-core attention kernel)
+    plain_layout: bool = False
 
     def page_tensors(self, page_size: int) -> dict[str, tuple[int, ...]]:
         k, d = self.n_kv_heads, self.head_dim
@@ -75,7 +83,8 @@ class PagedKVNeed(PagedNeed):
     def bind(self, group_id, tensors, page_size, dtype):
         from ..cache.pages import LayerPages, tiled_layout
 
-        return LayerPages(group_id, tensors["k"], tensors["v"], tiled_layout(dtype, self.head_dim, page_size))
+        tiled = not self.plain_layout and tiled_layout(dtype, self.head_dim, page_size)
+        return LayerPages(group_id, tensors["k"], tensors["v"], tiled)
 
 
 @dataclass(frozen=True)

@@ -10,6 +10,8 @@ per-request state, which the step function binds to every run of the layer.
 
 from __future__ import annotations
 
+import torch
+
 from ..kernels import ops
 from .base import FEED_FORWARDS, MIXERS, NORMS, Arrangement, register_arrangement
 from .norm import RMSNorm
@@ -94,4 +96,44 @@ class ParallelBlock(Arrangement):
         # both results are computed before either is added: both parts read the same stream
         self.mixer.forward(x, ctx, run, add_to=h)
         self.ff.forward(y, ctx, add_to=h)
+        return None
+
+
+@register_arrangement("post_norm")
+class PostNormBlock(Arrangement):
+    """``h = h + norm_a(mixer(h)); h = h + norm_b(ff(h))``: the parts read the stream itself
+    and the norm is on what they return.  A layer may leave the feed-forward (and its
+    norm) out.
+
+    The parts return float32 rows; norm, weight and sum are one float32 pass
+    (``ops.post_norm_add``), which also leaves the new rows rounded to the activation type
+    for the part that reads them next."""
+
+    graph_safe = True
+    roles = {"mixer": MIXERS, "mixer_norm": NORMS, "ff": FEED_FORWARDS, "ff_norm": NORMS}
+    optional = ("ff", "ff_norm")
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        self.mixer_norm, self.ff_norm, self.ff = parts["mixer_norm"], parts.get("ff_norm"), parts.get("ff")
+        if (self.ff is None) != (self.ff_norm is None):
+            raise ValueError("a post-norm block has a feed-forward and its norm, or neither")
+        for norm in (self.mixer_norm, self.ff_norm):
+            if norm is not None and not isinstance(norm, RMSNorm):
+                raise ValueError(f"a post-norm block norms with RMSNorm; {type(norm).__name__} is another")
+
+    def forward(self, h, pending, ctx, run):
+        if pending is not None:
+            ops.residual_add(h, pending)
+        dtype = self.mixer.build.dtype
+        a = self.mixer.forward(ops.cast_rows(h, dtype), ctx, run)
+        if a.dtype != torch.float32:
+            a = a.float()
+        x = ops.post_norm_add(h, a, self.mixer_norm.weight, self.mixer_norm.p.eps,
+                              cast_to=dtype if self.ff is not None else None)
+        if self.ff is not None:
+            b = self.ff.forward(x, ctx)
+            if b.dtype != torch.float32:
+                b = b.float()
+            ops.post_norm_add(h, b, self.ff_norm.weight, self.ff_norm.p.eps)
         return None

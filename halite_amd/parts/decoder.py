@@ -39,7 +39,8 @@ class Decoder:
     def __init__(self, spec: ModelSpec, dtype: torch.dtype, device: torch.device | str,
                  tiled_weights: bool = False):
         # the kinds of parts register themselves when their modules are imported
-        from . import attention, block, embedding, feedforward, latent_attention, moe, norm, rope  # noqa: F401
+        from . import (attention, block, embedding, feedforward, latent_attention, mixer_sum, moe, norm,  # noqa: F401
+                       normed_attention, rope, state_space)
 
         self.spec = spec
         self.dtype = dtype

@@ -3,6 +3,8 @@
 from __future__ import annotations
 
 import torch
+from typing import Literal
+
 from pydantic import BaseModel, Field, StrictInt, field_validator
 
 from ..kernels import ops
@@ -95,3 +97,35 @@ class GatedFeedForward(FeedForward):
         else:
             act = ops.silu_mul(ops.linear(x, w))
         return ops.linear(act, self.w_out, tiled=self.t_out, next_norm=then)
+
+
+class DenseParams(BaseModel):
+    hidden_size: StrictInt = Field(gt=0)
+    intermediate_size: StrictInt = Field(gt=0)
+    activation: Literal["relu_squared"] = "relu_squared"
+
+
+@FEED_FORWARDS.register("dense")
+class DenseFeedForward(FeedForward):
+    """``linear_out(act(linear_up(x)))`` without biases and without a gate; ``act`` is the
+    square of relu.  The result is float32 (the accumulators of the second product as they
+    are), for an arrangement that norms or adds it in float32."""
+
+    Params = DenseParams
+    graph_safe = True
+
+    def param_decls(self):
+        f, d = self.p.intermediate_size, self.p.hidden_size
+        return {"linear_up.weight": ParamDecl((f, d)), "linear_out.weight": ParamDecl((d, f))}
+
+    def finalize(self):
+        self.t_up = self.t_out = None
+        if self.build.tiled_weights and self.linear_up_weight.is_cuda and self.linear_up_weight.dtype == torch.bfloat16:
+            if self.p.hidden_size % 8 == 0:
+                self.t_up = ops.tile_weight(self.linear_up_weight)
+            if self.p.intermediate_size % 8 == 0 and self.linear_out_weight.dtype == torch.bfloat16:
+                self.t_out = ops.tile_weight(self.linear_out_weight)
+
+    def forward(self, x, ctx, then=None):
+        act = ops.relu_squared(ops.linear(x, self.linear_up_weight, tiled=self.t_up))
+        return ops.linear(act, self.linear_out_weight, out_dtype=torch.float32, tiled=self.t_out)

@@ -34,13 +34,25 @@ class BandedFrequencyScaling(BaseModel):
         return self
 
 
+class LinearFrequencyScaling(BaseModel):
+    """Every frequency divided by ``factor`` (positions stretched by it)."""
+
+    model_config = ConfigDict(extra="forbid")
+
+    kind: Literal["linear"]
+    factor: float = Field(gt=0)
+
+
 class RopeParams(BaseModel):
     head_dim: StrictInt = Field(gt=0)
     rotary_dim: StrictInt = Field(gt=0)
     theta: float = Field(gt=0)
     interleaved: StrictBool = False
     max_positions: StrictInt = Field(gt=0)
-    scaling: BandedFrequencyScaling | None = None
+    scaling: BandedFrequencyScaling | LinearFrequencyScaling | None = Field(default=None, discriminator="kind")
+    angles: Literal["float32", "float64"] = "float32"
+    """The arithmetic in which frequencies and angles are computed before cosine and sine
+    are rounded to the float32 table (float32: as the reference computes them)."""
 
     @model_validator(mode="after")
     def _check(self):
@@ -55,11 +67,14 @@ def rope_inverse_frequencies(p: RopeParams) -> torch.Tensor:
     ``original/low_freq_factor`` are stretched by ``factor``, shorter than
     ``original/high_freq_factor`` are kept, and between the two the stretched and
     the kept frequency are blended linearly in ``original/wavelength``."""
-    exponent = torch.arange(0, p.rotary_dim, 2, dtype=torch.float32, device="cpu") / p.rotary_dim
+    real = torch.float64 if p.angles == "float64" else torch.float32
+    exponent = torch.arange(0, p.rotary_dim, 2, dtype=real, device="cpu") / p.rotary_dim
     inv_freq = 1 / (p.theta**exponent)
     s = p.scaling
     if s is None:
         return inv_freq
+    if isinstance(s, LinearFrequencyScaling):
+        return inv_freq / s.factor
     long_wavelen = s.original_context_len / s.low_freq_factor
     short_wavelen = s.original_context_len / s.high_freq_factor
     wavelen = 2 * math.pi / inv_freq
@@ -101,8 +116,8 @@ class Rope(RotaryPositionEncoding):
         n = n_positions or self.p.max_positions
         if self._cos is None or self._cos.shape[0] < n:
             n = max(n, min(self.p.max_positions, 4096))
-            t = torch.arange(n, dtype=torch.float32, device="cpu")
+            t = torch.arange(n, dtype=self.inv_freq.dtype, device="cpu")
             angles = torch.outer(t, self.inv_freq)
-            self._cos = angles.cos().to(self.build.device).contiguous()
-            self._sin = angles.sin().to(self.build.device).contiguous()
+            self._cos = angles.cos().float().to(self.build.device).contiguous()
+            self._sin = angles.sin().float().to(self.build.device).contiguous()
         return self._cos, self._sin
