@@ -161,9 +161,36 @@ def chunked_attention(h, w, prefix, m, eps, fast=True):
     return o.reshape(T, -1) @ w[prefix + "o"].T
 
 
+def selective_scan(x, Bm, Cm, dt_raw, dt_bias, a_log, skip, S=None):
+    """``x`` [T, heads, P], ``Bm``, ``Cm`` [T, G, N], ``dt_raw`` [T, heads]; token by token
+    ``S <- exp(-exp(a_log) dt) S + dt B x^T`` and ``y = S^T C + skip x`` with
+    ``dt = softplus(dt_raw + dt_bias)``.  Returns ``y`` and the last state [heads, N, P]."""
+    T, heads, P = x.shape
+    G, N = Bm.shape[1:]
+    dt = softplus(dt_raw + dt_bias)
+    rate = torch.exp(a_log)
+    S = x.new_zeros(heads, N, P) if S is None else S.clone()
+    y = x.new_zeros(T, heads, P)
+    for t in range(T):
+        for hd in range(heads):
+            g = hd // (heads // G)
+            S[hd] = torch.exp(-rate[hd] * dt[t, hd]) * S[hd] + dt[t, hd] * torch.outer(Bm[t, g], x[t, hd])
+            y[t, hd] = S[hd].T @ Cm[t, g] + skip[hd] * x[t, hd]
+    return y, S
+
+
+def gated_part_norm(y, z, w, eps, parts):
+    """``y * silu(z)``, then every one of ``parts`` equal parts of a row divided by its own
+    root mean square, times ``w``."""
+    T, n = y.shape
+    y = (y * silu(z)).view(T, parts, n // parts)
+    y = y / torch.sqrt((y * y).mean(dim=-1, keepdim=True) + eps)
+    return y.reshape(T, n) * w
+
+
 def state_space(h, w, prefix, m, eps):
     """The right half of 'parallel': a selective state-space recurrence with scalar decay a
-    head, token by token."""
+    head."""
     T = h.shape[0]
     heads, P, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
     inner = heads * P
@@ -173,20 +200,8 @@ def state_space(h, w, prefix, m, eps):
     x = xbc[:, :inner].view(T, heads, P)
     Bm = xbc[:, inner : inner + G * N].view(T, G, N)
     Cm = xbc[:, inner + G * N :].view(T, G, N)
-    dt = softplus(dt + w[prefix + "dt_bias"])
-    rate = torch.exp(w[prefix + "A_log"])
-    S = h.new_zeros(heads, N, P)
-    y = h.new_zeros(T, heads, P)
-    for t in range(T):
-        for hd in range(heads):
-            g = hd // (heads // G)
-            S[hd] = torch.exp(-rate[hd] * dt[t, hd]) * S[hd] + dt[t, hd] * torch.outer(Bm[t, g], x[t, hd])
-            y[t, hd] = S[hd].T @ Cm[t, g] + w[prefix + "D"][hd] * x[t, hd]
-    y = y.reshape(T, inner) * silu(z)
-    parts = m["norm_groups"]
-    y = y.view(T, parts, inner // parts)
-    y = y / torch.sqrt((y * y).mean(dim=-1, keepdim=True) + eps)
-    y = y.reshape(T, inner) * w[prefix + "norm"]
+    y, _ = selective_scan(x, Bm, Cm, dt, w[prefix + "dt_bias"], w[prefix + "A_log"], w[prefix + "D"])
+    y = gated_part_norm(y.reshape(T, inner), z, w[prefix + "norm"], eps, m["norm_groups"])
     return y @ w[prefix + "o"].T
 
 
@@ -231,3 +246,122 @@ def read_model_folder(folder):
     with open(os.path.join(folder, "config.json")) as f:
         config = json.load(f)
     return config, load_file(os.path.join(folder, "model.safetensors"))
+
+
+# ---- small models of the tests' own ----------------------------------------------------------
+def attention_layer(heads, kv_heads, dim, scale, bias_max, coef, every, ff=None):
+    return dict(type="attention",
+                mixer=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=scale, bias_max=bias_max,
+                           q_temp=dict(coef=coef, every=every)),
+                mlp=None if ff is None else dict(kind="dense", ff=ff))
+
+
+def parallel_layer(left, right, left_scale, right_scale, ff=None):
+    return dict(type="parallel", mixer=dict(left=left, right=right, left_scale=left_scale, right_scale=right_scale),
+                mlp=None if ff is None else dict(kind="dense", ff=ff))
+
+
+def left_cfg(heads, kv_heads, dim, vdim, scale, conv, chunk, rot_dims, base=10000.0, factor=1.0):
+    return dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale, conv=conv, mask=dict(size=chunk),
+                rot=dict(base=base, dims=rot_dims, scaling=dict(factor=factor)))
+
+
+def right_cfg(heads, vdim, state, groups, conv, norm_groups):
+    return dict(heads=heads, vdim=vdim, state=state, groups=groups, conv=conv, norm_groups=norm_groups)
+
+
+def model_cfg(width, vocab, layers, eps=1e-5):
+    return dict(architecture="Zabunex", vocab=vocab, width=width, norm=dict(eps=eps), layers=layers)
+
+
+def tensor_shapes(cfg, bias_rows):
+    """Name -> shape of every tensor of a folder; ``bias_rows[i]``: rows of layer i's bias table."""
+    d = cfg["width"]
+    out = {"embed": (cfg["vocab"], d)}
+    for i, layer in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", layer["mixer"]
+        out[p + "norm1"] = (d,)
+        out[p + "norm2"] = (d,)
+        if layer["type"] == "attention":
+            nq, nk = m["heads"] * m["dim"], m["kv_heads"] * m["dim"]
+            out.update({p + "mix.q": (nq, d), p + "mix.k": (nk, d), p + "mix.q.norm": (nq,), p + "mix.k.norm": (nk,),
+                        p + "mix.rel": (bias_rows[i], m["heads"]), p + "mix.o": (d, m["heads"] * m["vdim"])})
+        else:
+            l, r = m["left"], m["right"]
+            nq, nk, nv = l["heads"] * l["dim"], l["kv_heads"] * l["dim"], l["kv_heads"] * l["vdim"]
+            q = p + "mix.left."
+            out.update({q + "q": (nq, d), q + "k": (nk, d), q + "v": (nv, d), q + "q.norm": (nq,), q + "k.norm": (nk,),
+                        q + "q.conv": (nq, l["conv"]), q + "k.conv": (nk, l["conv"]), q + "v.conv": (nv, l["conv"]),
+                        q + "o": (d, l["heads"] * l["vdim"])})
+            inner, gn = r["heads"] * r["vdim"], r["groups"] * r["state"]
+            q = p + "mix.right."
+            out.update({q + "in": (2 * inner + 2 * gn + r["heads"], d), q + "conv": (inner + 2 * gn, r["conv"]),
+                        q + "conv.b": (inner + 2 * gn,), q + "dt_bias": (r["heads"],), q + "A_log": (r["heads"],),
+                        q + "D": (r["heads"],), q + "norm": (inner,), q + "o": (d, inner)})
+        if layer.get("mlp") is not None:
+            out[p + "mlp.up"] = (layer["mlp"]["ff"], d)
+            out[p + "mlp.down"] = (d, layer["mlp"]["ff"])
+    out["final.norm"] = (d,)
+    out["head"] = (cfg["vocab"], d)
+    return out
+
+
+def random_weights(cfg, bias_rows, seed, std=0.12, stored=torch.bfloat16):
+    """Matrices N(0, std), norm weights around 1, bias tables and convolutions of a size that
+    counts, decays and step sizes spread over a range; rounded to ``stored`` so that engine
+    and plain model hold the same numbers."""
+    gen = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg, bias_rows).items():
+        last = name.rsplit(".", 1)[-1]
+        if last == "rel":
+            t = 1.5 * torch.randn(shape, generator=gen)
+        elif last == "conv":
+            t = 0.5 * torch.randn(shape, generator=gen)
+        elif last in ("b", "dt_bias"):
+            t = 0.5 * torch.randn(shape, generator=gen)
+        elif last == "A_log":
+            t = torch.rand(shape, generator=gen) * 2.0 - 2.0
+        elif len(shape) == 1:
+            t = 1.0 + 0.2 * torch.randn(shape, generator=gen)
+        else:
+            t = std * torch.randn(shape, generator=gen)
+        out[name] = t.to(stored).float()
+    return out
+
+
+def write_model_folder(folder, cfg, weights, dtype=torch.bfloat16):
+    from safetensors.torch import save_file
+
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.to(dtype).contiguous() for k, v in weights.items()}, os.path.join(folder, "model.safetensors"))
+    return folder
+
+
+# equal layers of each kind, grouped heads everywhere
+ZAB_A = model_cfg(64, 331, [
+    attention_layer(4, 2, 16, 0.25, 40, 0.3, 16, ff=96),
+    parallel_layer(left_cfg(4, 2, 16, 16, 0.25, 3, 24, 8, factor=2.0), right_cfg(4, 16, 16, 2, 4, 2), 0.7, 1.2, ff=80),
+    attention_layer(4, 2, 16, 0.25, 40, 0.3, 16, ff=96),
+])
+ZAB_A_BIAS = {0: 12, 2: 12}
+# the recurrent layer first; value heads of another size than the keys', one group, one
+# norm part, a temperature that changes with every position, chunks shorter than a page, a
+# rotation of the whole head without stretching, a layer without a feed-forward
+ZAB_B = model_cfg(48, 257, [
+    parallel_layer(left_cfg(2, 1, 24, 8, 0.2, 2, 7, 24, base=500.0), right_cfg(3, 8, 8, 1, 2, 1), 1.0, -0.5),
+    attention_layer(6, 2, 8, 0.35, 17, -0.2, 1, ff=64),
+    parallel_layer(left_cfg(4, 4, 8, 24, 0.3, 4, 33, 2, factor=4.0), right_cfg(2, 24, 16, 2, 3, 4), 0.4, 0.9, ff=40),
+])
+ZAB_B_BIAS = {1: 10}
+# sizes that are multiples of little: head sizes that pages pad, a state of 24 numbers, a
+# convolution of one tap and one of five, a chunk of exactly a page, a single bias row per
+# distance up to the table's half
+ZAB_C = model_cfg(40, 199, [
+    attention_layer(3, 3, 20, 0.22, 100, 0.5, 64, ff=52),
+    parallel_layer(left_cfg(3, 3, 12, 20, 0.29, 5, 16, 4, base=1.0e6, factor=8.0), right_cfg(5, 12, 24, 5, 1, 3), 0.6, 1.1, ff=36),
+    attention_layer(2, 1, 12, 0.3, 9, 0.0, 5),
+])
+ZAB_C_BIAS = {0: 6, 2: 16}
