@@ -115,7 +115,10 @@ __device__ __forceinline__ void load_to_lds(const bf16_t* src, void* lds) {
 // Two waves per SIMD leave 256 registers each, which keeps the accumulators in VGPRs (no
 // copies to and from AGPRs around every MFMA); the largest head sizes need more.
 #define MIN_WAVES_PER_SIMD (D > 160 ? 1 : 2)
-template <int RT, bool POW2, bool PAGE32, bool SHARED, bool TILED, int KB, int HALVES>
+// RULED: the scores follow a rule beyond scale, causal mask and window (`hal_score_rule`): a
+// bias by distance (the table comes multiplied by log2 e), a sink in the denominator; a
+// chunked mask needs no build of its own.
+template <int RT, bool POW2, bool PAGE32, bool SHARED, bool TILED, int KB, int HALVES, bool RULED>
 __global__ void __launch_bounds__(256 * HALVES, MIN_WAVES_PER_SIMD)
 attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
                       int out_row_stride, const int* __restrict__ items,
@@ -125,7 +128,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
                       const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                       float* __restrict__ part_o, float* __restrict__ part_ml,
                       int* __restrict__ counters, int H, int K, int page_size, int page_shift,
-                      float scale_log2e, int window, int max_items) {
+                      float scale_log2e, hal_score_rule rule, int max_items) {
   static_assert(HALVES == 1 || (SHARED && HALVES == 2), "only the kernel with LDS has two halves");
   // JOIN (the kernel without LDS for keys): the four items of a workgroup are four pieces of
   // one tile's key range (the host lists them so, in whole runs of four, the last may be
@@ -240,7 +243,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     qi[rt] = row_ok[rt] ? rho / G : 0;
     head[rt] = g * G + (row_ok[rt] ? rho % G : 0);
     p_row[rt] = pos0 + qi[rt];  // the row's position: it sees keys <= p_row
-    lo_row[rt] = (window > 0 && p_row[rt] - window + 1 > 0) ? p_row[rt] - window + 1 : 0;
+    lo_row[rt] = hal_rule_lo(rule, p_row[rt]);
     const bf16_t* qp = q + (size_t)(q_start + qi[rt]) * q_row_stride + (size_t)head[rt] * D;
 #pragma unroll
     for (int ks = 0; ks < KT; ++ks) {
@@ -268,8 +271,8 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     if (r_last < r_first) r_last = r_first;
     p_first[rt] = pos0 + r_first / G;
     p_last[rt] = r_first >= 0 ? pos0 + r_last / G : -1;  // no tile: no key is in range
-    lo_first[rt] = (window > 0 && p_first[rt] - window + 1 > 0) ? p_first[rt] - window + 1 : 0;
-    lo_last[rt] = (window > 0 && p_last[rt] - window + 1 > 0) ? p_last[rt] - window + 1 : 0;
+    lo_first[rt] = hal_rule_lo(rule, p_first[rt] > 0 ? p_first[rt] : 0);
+    lo_last[rt] = hal_rule_lo(rule, p_last[rt] > 0 ? p_last[rt] : 0);
   }
 
   // This lane's key of tile t in the block of 32 keys at j0: row `col` of tile t is
@@ -371,10 +374,21 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       float m_raw = -INFINITY;
       const bool full = j0 >= kv_begin && j0 + KB <= kv_end && j0 + KB - 1 <= p_first[rt] &&
                         j0 >= lo_last[rt];
+      // (RULED: sv holds scaled scores, in units of log2, with the bias added)
+      auto ruled = [&](float raw, int j) {
+        if constexpr (RULED) {
+          if (rule.bias == nullptr) return raw * scale_log2e;
+          int back = p_row[rt] - j;
+          back = back < 0 ? 0 : (back < rule.bias_len ? back : rule.bias_len - 1);
+          return __builtin_fmaf(raw, scale_log2e, rule.bias[(size_t)head[rt] * rule.bias_len + back]);
+        } else {
+          return raw;
+        }
+      };
       if (full) {  // every key of the step is visible to every row of the tile
 #pragma unroll
         for (int e = 0; e < SUBS * 8; ++e) {
-          sv[e] = s[rt][e / 8][(e % 8) / 4][e % 4];
+          sv[e] = ruled(s[rt][e / 8][(e % 8) / 4][e % 4], j0 + (e / 8) * 32 + quad * 8 + e % 8);
           m_raw = fmaxf(m_raw, sv[e]);
         }
       } else {
@@ -383,12 +397,12 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
           const int j = j0 + (e / 8) * 32 + quad * 8 + e % 8;
           const bool ok =
               row_ok[rt] && j >= kv_begin && j < kv_end && j >= lo_row[rt] && j <= p_row[rt];
-          sv[e] = ok ? s[rt][e / 8][(e % 8) / 4][e % 4] : -INFINITY;
+          sv[e] = ok ? ruled(s[rt][e / 8][(e % 8) / 4][e % 4], j) : -INFINITY;
           m_raw = fmaxf(m_raw, sv[e]);
         }
       }
       m_raw = max_across_16(max_across_32(m_raw));
-      const float m_tile = m_raw * scale_log2e;
+      const float m_tile = RULED ? m_raw : m_raw * scale_log2e;
       // The running maximum only has to keep exp2(s - m) in range, so it is raised
       // only when the step's maximum exceeds it by more than 2^RESCALE_SLACK: then
       // the accumulated sums are rarely rescaled (and a partial result's m, l and sums
@@ -402,7 +416,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       float psum = 0.f;
 #pragma unroll
       for (int e = 0; e < SUBS * 8; ++e) {
-        pv[e] = fast_exp2(__builtin_fmaf(sv[e], scale_log2e, -m_sub));
+        pv[e] = RULED ? fast_exp2(sv[e] - m_sub) : fast_exp2(__builtin_fmaf(sv[e], scale_log2e, -m_sub));
         psum += pv[e];
       }
       l[rt] = l[rt] * alpha[rt] + psum;
@@ -851,6 +865,9 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     }
     if (!row_ok[rt]) continue;
     if (partial < 0 || merged_here) {
+      if constexpr (RULED) {
+        if (rule.sink && m[rt] != -INFINITY) lt += exp2f(-m[rt]);  // (sums are relative to 2^m)
+      }
       const float inv = lt > 0.f ? 1.0f / lt : 0.f;
       bf16_t* op = out + (size_t)(q_start + qi[rt]) * out_row_stride + (size_t)head[rt] * D;
 #pragma unroll
@@ -883,7 +900,7 @@ __global__ void __launch_bounds__(256)
 attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
                        const int* __restrict__ merges, const int* __restrict__ n_merges_ptr,
                        const float* __restrict__ part_o, const float* __restrict__ part_ml, int H,
-                       int K) {
+                       int K, int sink) {
   constexpr int NC = (D + 127) / 128;  // a lane's pairs of dimensions
   constexpr int MW = 4;                // waves
   __shared__ float red_o[MW][NC * 128];
@@ -955,6 +972,7 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
   float l_sum = 0.f;
 #pragma unroll
   for (int w = 0; w < MW; ++w) l_sum += red_l[w];
+  if (sink && m_all != -INFINITY) l_sum += exp2f(-m_all);
   const float inv = l_sum > 0.f ? 1.0f / l_sum : 0.f;
   const int qi = rho / G, head = g * G + rho % G;
   bf16_t* op = out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D;
@@ -979,7 +997,7 @@ __global__ void __launch_bounds__(256)
 attention_merge_few_kernel(bf16_t* __restrict__ out, int out_row_stride,
                            const int* __restrict__ merges, const int* __restrict__ n_merges_ptr,
                            const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                           int H, int K) {
+                           int H, int K, int sink) {
   constexpr int NC = (D + 127) / 128;
   const int mi = blockIdx.x;
   const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
@@ -1011,6 +1029,7 @@ attention_merge_few_kernel(bf16_t* __restrict__ out, int out_row_stride,
       acc[c][1] += w * v.y;
     }
   }
+  if (sink && m_all != -INFINITY) l_all += exp2f(-m_all);
   const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
   const int qi = rho / G, head = g * G + rho % G;
   bf16_t* op = out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D;
@@ -1061,6 +1080,31 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
                                   int* counters, int n_counters, int H, int K, int head_dim,
                                   int page_size, int tiled, float scale, int window,
                                   int merge_parts, hipStream_t stream) {
+  return hal_attention_mfma_ruled(q, q_row_stride, out, out_row_stride, items, max_items, big_items,
+                                  max_big, merges, max_merges, counts, seg_q_start, seg_q_len,
+                                  seg_kv_len, block_table, bt_stride, k_pages, v_pages, part_o, part_ml,
+                                  counters, n_counters, H, K, head_dim, page_size, tiled, scale, window,
+                                  0, nullptr, 0, 0, merge_parts, stream);
+}
+
+// The same with a rule for the scores.  `chunk`: the work lists must have been cut for it (a
+// tile's first key is no earlier than the start of its first row's chunk).  `bias_log2`:
+// float32 [H][bias_len], the bias by distance times log2 e.
+extern "C" int hal_attention_mfma_ruled(const void* q, int q_row_stride, void* out, int out_row_stride,
+                                        const int* items, int max_items, const int* big_items,
+                                        int max_big, const int* merges, int max_merges,
+                                        const int* counts, const int* seg_q_start,
+                                        const int* seg_q_len, const int* seg_kv_len,
+                                        const int* block_table, int bt_stride, const void* k_pages,
+                                        const void* v_pages, float* part_o, float* part_ml,
+                                        int* counters, int n_counters, int H, int K, int head_dim,
+                                        int page_size, int tiled, float scale, int window, int chunk,
+                                        const float* bias_log2, int bias_len, int sink,
+                                        int merge_parts, hipStream_t stream) {
+  HAL_REQUIRE(chunk >= 0 && (bias_log2 == nullptr || bias_len > 0),
+              "hal_attention_mfma: chunk %d, bias table of %d distances", chunk, bias_len);
+  const hal_score_rule rule = {window, chunk, bias_len, sink ? 1 : 0, bias_log2};
+  const bool ruled = bias_log2 != nullptr || sink;
   HAL_REQUIRE(head_dim == D, "hal_attention_mfma: built for head size %d, called with %d", D,
               head_dim);
   HAL_REQUIRE(H > 0 && K > 0 && H % K == 0, "hal_attention_mfma: %d heads, %d kv heads", H, K);
@@ -1084,15 +1128,20 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
 #define LAUNCH_ATTENTION(RT_, SHARED_, KB_, HV_, LIST, MAX, COUNT)                                 \
   {                                                                                               \
     dim3 grid(((MAX) + waves - 1) / waves, K);                                                    \
-    auto kernel = attention_mfma_kernel<RT_, false, false, SHARED_, false, KB_, HV_>;             \
-    if (tiled) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, D % 32 == 0, KB_, HV_>;   \
-    else if (page_shift >= 5) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, false, KB_, HV_>; \
-    else if (page_shift >= 0) kernel = attention_mfma_kernel<RT_, true, false, SHARED_, false, KB_, HV_>; \
+    auto kernel = attention_mfma_kernel<RT_, false, false, SHARED_, false, KB_, HV_, false>;      \
+    if (ruled) {                                                                                  \
+      kernel = attention_mfma_kernel<RT_, false, false, SHARED_, false, KB_, HV_, true>;          \
+      if (tiled) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, D % 32 == 0, KB_, HV_, true>; \
+      else if (page_shift >= 5) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, false, KB_, HV_, true>; \
+      else if (page_shift >= 0) kernel = attention_mfma_kernel<RT_, true, false, SHARED_, false, KB_, HV_, true>; \
+    } else if (tiled) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, D % 32 == 0, KB_, HV_, false>; \
+    else if (page_shift >= 5) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, false, KB_, HV_, false>; \
+    else if (page_shift >= 0) kernel = attention_mfma_kernel<RT_, true, false, SHARED_, false, KB_, HV_, false>; \
     hipLaunchKernelGGL(kernel, grid, dim3(waves * HAL_WAVE * HV_), 0, stream, (const bf16_t*)q,   \
                        q_row_stride, (bf16_t*)out, out_row_stride, LIST, COUNT, seg_q_start,      \
                        seg_q_len, seg_kv_len, block_table, bt_stride, (const bf16_t*)k_pages,     \
                        (const bf16_t*)v_pages, part_o, part_ml, counters, H, K, page_size,        \
-                       page_shift, scale_log2e, window, MAX);                                     \
+                       page_shift, scale_log2e, rule, MAX);                                       \
     HAL_LAUNCH_CHECK();                                                                           \
   }
   HAL_REQUIRE(max_items % WAVES == 0 && max_big % WAVES == 0,
@@ -1106,10 +1155,12 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
   if (max_merges > 0) {
     if (merge_parts > 0 && merge_parts <= MERGE_FEW_PARTS)
       hipLaunchKernelGGL(attention_merge_few_kernel, dim3(max_merges, K, 4), dim3(256), 0, stream,
-                         (bf16_t*)out, out_row_stride, merges, counts + 2, part_o, part_ml, H, K);
+                         (bf16_t*)out, out_row_stride, merges, counts + 2, part_o, part_ml, H, K,
+                         rule.sink);
     else
       hipLaunchKernelGGL(attention_merge_kernel, dim3(max_merges, K, 16), dim3(256), 0, stream,
-                         (bf16_t*)out, out_row_stride, merges, counts + 2, part_o, part_ml, H, K);
+                         (bf16_t*)out, out_row_stride, merges, counts + 2, part_o, part_ml, H, K,
+                         rule.sink);
     HAL_LAUNCH_CHECK();
   }
   return 0;

@@ -252,4 +252,16 @@ int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_s
                        int n_counters, int H, int K, int head_dim, int page_size, int tiled,
                        float scale, int window, int merge_parts, hipStream_t stream);
 
+// hal_attention_mfma with a rule for the scores (see hal_attention_simple_ruled); the bias
+// table comes multiplied by log2 e, and the work lists are cut for the chunk.
+int hal_attention_mfma_ruled(const void* q, int q_row_stride, void* out, int out_row_stride,
+                             const int* items, int max_items, const int* big_items, int max_big,
+                             const int* merges, int max_merges, const int* counts,
+                             const int* seg_q_start, const int* seg_q_len, const int* seg_kv_len,
+                             const int* block_table, int bt_stride, const void* k_pages,
+                             const void* v_pages, float* part_o, float* part_ml, int* counters,
+                             int n_counters, int H, int K, int head_dim, int page_size, int tiled,
+                             float scale, int window, int chunk, const float* bias_log2,
+                             int bias_len, int sink, int merge_parts, hipStream_t stream);
+
 }  // extern "C"

@@ -184,15 +184,15 @@ class StepContext:
     # The plans of the attention kernel are part of the same upload, so they are
     # declared before the first device access.
     def plan_attention(self, group_id: int, n_heads: int, n_kv_heads: int, window: int,
-                       head_dim: int, late=False) -> None:
-        key = (group_id, n_heads // n_kv_heads, window)
+                       head_dim: int, late=False, chunk: int = 0) -> None:
+        key = (group_id, n_heads // n_kv_heads, window, chunk)
         if key in self._plan_host:
             return
         if self._dev is not None and not late:
             return
         plan = attention_kernels.plan_items(
             self.seg_q_len_host, self.seg_kv_len_host, n_heads // n_kv_heads, n_kv_heads, window,
-            attention_kernels.rows_per_big_item(head_dim),
+            attention_kernels.rows_per_big_item(head_dim), chunk,
         )
         self._plan_host[key] = plan
         plan.name = f"plan{len(self._plan_host)}"
@@ -257,8 +257,8 @@ class StepContext:
         (``kernels.ops.ScoreRule``): a chunked mask, a bias by distance, a sink."""
         return attention_kernels.paged_attention(self, q, q_row_stride, kv, group, n_heads, scale, window, rule)
 
-    def device_plan(self, group_id: int, group_size: int, window: int):
-        key = (group_id, group_size, window)
+    def device_plan(self, group_id: int, group_size: int, window: int, chunk: int = 0):
+        key = (group_id, group_size, window, chunk)
         plan = self._plan_host.get(key)
         if plan is None:
             return None

@@ -150,9 +150,10 @@ def rows_per_big_item(head_dim: int) -> int:
     return int(library.attention_library(head_dim).hal_attention_mfma_rows_per_big_item())
 
 
-def _tiles(seg_q_len, seg_kv_len, group_size, window, rows_per_tile, pick):
+def _tiles(seg_q_len, seg_kv_len, group_size, window, rows_per_tile, pick, chunk=0):
     """The tiles of ``rows_per_tile`` rows of the segments whose row count ``pick``
-    accepts: segment, first row, first and end key of each (arrays)."""
+    accepts: segment, first row, first and end key of each (arrays).  ``chunk``: a row sees
+    no key before the start of its own chunk of that many positions."""
     ql = np.asarray(seg_q_len, dtype=np.int64)
     kl = np.asarray(seg_kv_len, dtype=np.int64)
     rows = ql * group_size
@@ -168,6 +169,8 @@ def _tiles(seg_q_len, seg_kv_len, group_size, window, rows_per_tile, pick):
     last_q = np.minimum(rows[seg_ids] - 1, r0 + rows_per_tile - 1) // group_size
     pos0 = (kl - ql)[seg_ids]
     b = np.zeros_like(r0) if window <= 0 else np.maximum(0, pos0 + first_q - window + 1)
+    if chunk > 0:
+        b = np.maximum(b, (pos0 + first_q) // chunk * chunk)
     e = pos0 + last_q + 1
     return seg_ids, r0, b, e
 
@@ -328,7 +331,7 @@ def _group_tiles(seg_ids, rho0s, kv_b, kv_e, per_item: int):
 
 
 def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: int,
-               rows_big: int = 64) -> AttentionPlan:
+               rows_big: int = 64, chunk: int = 0) -> AttentionPlan:
     """Cuts the step's query rows into tiles of 16 rows.  A segment of at most 16 rows or
     of one token (decode tokens) gives one-tile items, four to a workgroup, which takes a
     piece of the tile's key range; a longer segment gives items of ``rows_big / 16`` tiles
@@ -340,8 +343,8 @@ def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: 
     # (a single token is never a long segment, however many heads share its keys: a decode
     # step then has one-tile items only, whose room is known before the lengths are)
     short = lambda r, q: (r <= ROWS_PER_ITEM) | (q == 1) | (per_item == 1)
-    small = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, short)
-    big = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r, q: ~short(r, q))
+    small = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, short, chunk)
+    big = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r, q: ~short(r, q), chunk)
     items, merges_s, slot = _cut_joined(*small, pieces_per_tile(len(small[0]), n_kv_heads), 0, seg_scalars)
     more = None
     if len(big[0]):
@@ -392,7 +395,7 @@ def counters_idle(device) -> bool:
     return key not in _COUNTERS or int(_COUNTERS[key].abs().sum()) == 0
 
 
-def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, window):
+def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, window, rule=None):
     plan, items, big_items, merges, counts = plan_dev
     n_pages, n_kv, page_size, head_dim = kv.k.shape
     lib = library.attention_library(head_dim)
@@ -405,13 +408,20 @@ def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, wi
     if plan.merged_in_kernel:
         counters = _counters(q.device)
     P = ops._ptr
-    rc = lib.hal_attention_mfma(
+    rule = rule or ops.ScoreRule()
+    bias = rule.bias_log2 if rule.bias is not None else None
+    if rule.bias is not None:
+        ops._need(bias is not None and bias.is_cuda and bias.is_contiguous() and bias.dtype == torch.float32
+                  and bias.dim() == 2 and bias.shape[0] == n_heads and bias.shape == rule.bias.shape,
+                  "attention: the bias times log2 e is float32 [heads, distances]")
+    rc = lib.hal_attention_mfma_ruled(
         P(q), q_row_stride, P(out), n_heads * head_dim,
         P(items), plan.cap_items, P(big_items), plan.cap_big, P(merges), plan.cap_merges, P(counts),
         P(ctx.seg_q_start), P(ctx.seg_q_len), P(ctx.seg_kv_len),
         P(group.block_table), group.block_table.shape[1], P(kv.k), P(kv.v), P(part_o), P(part_ml),
         P(counters), N_COUNTERS, n_heads, n_kv, head_dim, page_size, 1 if getattr(kv, "tiled", False) else 0,
-        ctypes.c_float(scale), window, plan.max_parts, ops._stream(),
+        ctypes.c_float(scale), window, rule.chunk, P(bias), 0 if bias is None else bias.shape[1],
+        1 if rule.sink else 0, plan.max_parts, ops._stream(),
     )
     ops._check(lib, rc)
     return out
@@ -425,13 +435,13 @@ def upload_plan(plan: AttentionPlan, device):
 
 def paged_attention(ctx, q, q_row_stride, kv, group, n_heads, scale, window, rule=None):
     n_pages, n_kv, page_size, head_dim = kv.k.shape
-    ruled = rule is not None and not rule.plain()
-    if not ruled and mfma_supported(q.dtype, head_dim, page_size) and q_row_stride % 8 == 0:
-        plan_dev = ctx.device_plan(group.group_id, n_heads // n_kv, window)
+    chunk = rule.chunk if rule is not None else 0
+    if mfma_supported(q.dtype, head_dim, page_size) and q_row_stride % 8 == 0:
+        plan_dev = ctx.device_plan(group.group_id, n_heads // n_kv, window, chunk)
         if plan_dev is None:
-            ctx.plan_attention(group.group_id, n_heads, n_kv, window, head_dim, late=True)
-            plan_dev = ctx.device_plan(group.group_id, n_heads // n_kv, window)
-        return attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, window)
+            ctx.plan_attention(group.group_id, n_heads, n_kv, window, head_dim, late=True, chunk=chunk)
+            plan_dev = ctx.device_plan(group.group_id, n_heads // n_kv, window, chunk)
+        return attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, window, rule)
     if getattr(kv, "tiled", False):
         raise ops.KernelError(
             f"pages are kept in the matrix-core kernel's order, which only that kernel reads "

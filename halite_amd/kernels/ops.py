@@ -35,6 +35,8 @@ class ScoreRule:
     chunk: int = 0
     bias: torch.Tensor | None = None
     sink: bool = False
+    # the same table times log2 e, for the kernel whose exponentials are to the base 2
+    bias_log2: torch.Tensor | None = None
 
     def plain(self) -> bool:
         return self.chunk == 0 and self.bias is None and not self.sink

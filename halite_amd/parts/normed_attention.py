@@ -21,6 +21,8 @@ of 16), the rest zero.  The result is float32 (the accumulators of the output pr
 
 from __future__ import annotations
 
+import math
+
 import numpy as np
 import torch
 from pydantic import BaseModel, Field, StrictBool, StrictInt, model_validator
@@ -167,14 +169,20 @@ class NormedAttention(Mixer):
             rows = torch.from_numpy(distance_buckets(p.distance_bias.buckets, p.distance_bias.max_distance))
             table = self.w_distance_bias.float()[rows.to(self.w_distance_bias.device)]
             self.bias_table = table.t().contiguous()
-        self.rule = ops.ScoreRule(chunk=p.chunk or 0, bias=self.bias_table, sink=p.sink)
+        self.rule = ops.ScoreRule(
+            chunk=p.chunk or 0, bias=self.bias_table, sink=p.sink,
+            bias_log2=None if self.bias_table is None else (self.bias_table.double() * math.log2(math.e)).float().contiguous(),
+        )
 
     def cache_need(self):
         p = self.p
-        return PagedKVNeed(p.n_kv_heads, self.head_dim, p.window, p.chunk, plain_layout=not self._on_matrix_cores())
+        return PagedKVNeed(p.n_kv_heads, self.head_dim, p.window, p.chunk)
 
-    def _on_matrix_cores(self) -> bool:
-        return False
+    def prepare(self, ctx, run):
+        group = ctx.cache.groups[run.kv.group_id]
+        if attention_kernels.mfma_supported(self.build.dtype, self.head_dim, group.page_size):
+            ctx.plan_attention(group.group_id, self.p.n_heads, self.p.n_kv_heads, self.p.window or 0, self.head_dim,
+                               chunk=self.p.chunk or 0)
 
     def state_need(self):
         if self.p.conv_taps is None or self.p.conv_taps == 1:
