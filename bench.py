@@ -99,7 +99,9 @@ class Families:
     GEMM = ("linear", "linear_add", "gemm_bf16_skinny", "gemm_bf16_skinny_norm", "qkv_rope_append", "gemm_f32")
     GROUPED = ("grouped_gemm",)
     ELEMENTWISE = ("rmsnorm", "silu_mul", "rope_append", "embedding", "residual_add", "rmsnorm_exact", "latent_prep",
-                   "head_cols", "scale_", "moe_route", "moe_sort", "moe_combine", "clamped_gate_mul")
+                   "head_cols", "scale_", "moe_route", "moe_sort", "moe_combine", "clamped_gate_mul", "cast_rows",
+                   "post_norm_add", "relu_squared", "scaled_sum_", "qk_norm_pack", "gated_part_norm")
+    RECURRENT = ("short_conv", "short_conv_carry", "ssd_scan")
 
     def __init__(self):
         self.spans = []
@@ -137,6 +139,8 @@ class Families:
             self._wrap(ops, name, "grouped")
         for name in self.ELEMENTWISE:
             self._wrap(ops, name, "elementwise")
+        for name in self.RECURRENT:
+            self._wrap(ops, name, "recurrent")
         self._wrap(attention_kernels, "paged_attention", "attention")
         return self
 
@@ -357,14 +361,85 @@ def llama_work(c, n_layers, tokens, batch=0, kv_tokens=0) -> dict:
             "attention": 2.0 * n_layers * kv_tokens * 2 * c.num_key_value_heads * c.head_dim}
 
 
+# Layers of the Zabunex design at two sizes that resemble served models: three layers of the
+# attention with a bias by distance and one of the chunked attention beside the state-space
+# mixer to every four, as many weights in the feed-forward's two matrices as in the three of
+# the Llama layer beside it (same width, heads, head size and grouping).
+ZABUNEX_SIZES = {
+    "2048-wide": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=12288, llama_ff=8192, chunk=1024, bias_max=2048,
+                      ssm_heads=32, ssm_dim=64, state=128, groups=8),
+    "4096-wide": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=21504, llama_ff=14336, chunk=1024, bias_max=2048,
+                      ssm_heads=64, ssm_dim=64, state=128, groups=8),
+}
+
+
+def zabunex_layer_kinds(n_layers):
+    return ["parallel" if i % 4 == 3 else "attention" for i in range(n_layers)]
+
+
+def zabunex_config(s, n_layers, window):
+    attention = dict(heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["dim"], scale=s["dim"] ** -0.5,
+                     bias_max=s["bias_max"], bias_buckets=32, q_temp=dict(coef=0.1, every=1024))
+    left = dict(heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["dim"], scale=s["dim"] ** -0.5, conv=4,
+                mask=dict(size=s["chunk"]), rot=dict(base=500000.0, dims=64, scaling=dict(factor=8.0)))
+    right = dict(heads=s["ssm_heads"], vdim=s["ssm_dim"], state=s["state"], groups=s["groups"], conv=4, norm_groups=s["groups"])
+    mlp = dict(kind="dense", ff=s["ff"])
+    layers = [dict(type="attention", mixer=attention, mlp=mlp) if kind == "attention" else
+              dict(type="parallel", mixer=dict(left=left, right=right, left_scale=0.6, right_scale=1.1), mlp=mlp)
+              for kind in zabunex_layer_kinds(n_layers)]
+    return dict(architecture="Zabunex", vocab=COMPARISON_VOCAB, width=s["width"], norm=dict(eps=1e-5), max_positions=8192,
+                layers=layers)
+
+
+def llama_beside_zabunex(s, n_layers):
+    return dict(LLAMA_3_1_8B, vocab_size=COMPARISON_VOCAB, hidden_size=s["width"], num_hidden_layers=n_layers,
+                num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"], head_dim=s["dim"],
+                intermediate_size=s["llama_ff"], max_position_embeddings=8192, rope_scaling=None)
+
+
+def zabunex_work(s, n_layers, tokens, batch=0, kv_tokens=0, elt=2) -> dict:
+    """As ``kavuvik_work``; the family ``recurrent`` is the convolutions and the recurrence,
+    float32 arithmetic on the vector units (counted against their peak) whose decode step
+    reads and writes the float32 state of every request."""
+    d, h, kv, D = s["width"], s["heads"], s["kv_heads"], s["dim"]
+    kinds = zabunex_layer_kinds(n_layers)
+    n_att, n_par = kinds.count("attention"), kinds.count("parallel")
+    inner, gn = s["ssm_heads"] * s["ssm_dim"], s["groups"] * s["state"]
+    att = d * (h + kv) * D + h * D * d
+    par = d * (h + 2 * kv) * D + h * D * d + d * (2 * inner + 2 * gn + s["ssm_heads"]) + inner * d
+    ff = 2 * d * s["ff"]
+    linear = n_att * att + n_par * par + n_layers * ff
+    state = s["ssm_heads"] * s["state"] * s["ssm_dim"]
+    if batch == 0:
+        seen = min(tokens, s["chunk"])  # the keys a chunked layer's token sees at most
+        return {"gemm": 2.0 * tokens * linear + 2.0 * COMPARISON_VOCAB * d,
+                "attention": 2.0 * tokens * h * D * (tokens * n_att + seen * n_par),
+                "recurrent": tokens * n_par * (6.0 * state + 8.0 * ((h + 2 * kv) * D + inner + 2 * gn))}
+    per_request = kv_tokens / batch
+    return {"gemm": 2.0 * (linear + COMPARISON_VOCAB * d),
+            "attention": 2.0 * 2 * kv * D * (kv_tokens * n_att + batch * (per_request % s["chunk"]) * n_par),
+            "recurrent": 2.0 * batch * n_par * 2 * state * 4 / elt}
+
+
+DESIGNS = {
+    "kavuvik": dict(label="Kavuvik", sizes=lambda: KAVUVIK_SIZES, config=lambda s, n, w: kavuvik_config(s, n, w),
+                    llama=lambda s, n: closest_llama_config(s, n),
+                    work=lambda s, n, t, b, kv, elt: kavuvik_work(s, n, t, b, kv)),
+    "zabunex": dict(label="Zabunex", sizes=lambda: ZABUNEX_SIZES, config=lambda s, n, w: zabunex_config(s, n, w),
+                    llama=lambda s, n: llama_beside_zabunex(s, n),
+                    work=lambda s, n, t, b, kv, elt: zabunex_work(s, n, t, b, kv, elt)),
+}
+
+
 def design_comparison(args) -> dict:
-    """``--workload kavuvik``: prefill and decode throughput of Kavuvik layers at two sizes
-    beside the closest Llama layers, with each family of kernels against its roofline (the
-    products and the attention of a prompt against the bf16 matrix peak, those of a decode
-    step against the memory's bandwidth).  Random weights; a few layers each, named in the record."""
+    """``--workload kavuvik`` / ``zabunex``: prefill and decode throughput of the design's
+    layers at two sizes beside the closest Llama layers, with each family of kernels against
+    its roofline (the products and the attention of a prompt against the bf16 matrix peak, a
+    recurrence against the float32 vector peak, those of a decode step against the memory's
+    bandwidth).  Random weights; a few layers each, named in the record."""
     import torch
 
-    from halite_amd.config import KavuvikConfig, LlamaConfig, ModelConfig, ServerConfig
+    from halite_amd.config import LlamaConfig, ModelConfig, ServerConfig, parse_config
     from halite_amd.engine.batch import Segment
     from halite_amd.engine.runner import ModelRunner
 
@@ -372,6 +447,9 @@ def design_comparison(args) -> dict:
     prompt, context, batches = args.prefill_tokens, args.context or 2048, (8, 64)
     gen = torch.Generator().manual_seed(0)
     peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+    peak_of = lambda family: PEAK_FLOPS["fp32"] if family == "recurrent" else peak  # noqa: E731
+    design = DESIGNS[args.workload]
+    label = design["label"]
 
     def best_ms(fn, reps):
         times = []
@@ -411,7 +489,7 @@ def design_comparison(args) -> dict:
         out["prefill"] = {"tokens": prompt, "ms": round(ms, 3), "tok_per_s": round(prompt / ms * 1e3, 1),
                           "of_peak": round(sum(flops.values()) / (ms * 1e-3) / peak, 4),
                           "families_ms": {k: round(v, 3) for k, v in by.items()},
-                          "families_of_peak": {k: round(flops[k] / (by[k] * 1e-3) / peak, 4) for k in flops if by.get(k)}}
+                          "families_of_peak": {k: round(flops[k] / (by[k] * 1e-3) / peak_of(k), 4) for k in flops if by.get(k)}}
         out["decode"] = {}
         for b in batches:
             slots = [runner.admit() for _ in range(b)]
@@ -439,7 +517,7 @@ def design_comparison(args) -> dict:
                 by = fam.totals_ms()
             runner.graphs_allowed = graphs
             elt = 2 if args.dtype == "bfloat16" else 4
-            bytes_ = {k: v / 2 * elt for k, v in work(0, b, b * pos[0]).items()}
+            bytes_ = {k: v / 2 * elt for k, v in work(0, b, b * pos[0], elt).items()}
             out["decode"][f"batch{b}"] = {
                 "context": pos[0], "ms_per_step": round(ms, 4), "tok_per_s": round(b / ms * 1e3, 1),
                 "of_bandwidth": round(sum(bytes_.values()) / (ms * 1e-3) / HBM_BYTES_PER_S, 4),
@@ -451,24 +529,25 @@ def design_comparison(args) -> dict:
         return out
 
     sizes = {}
-    for name, s in KAVUVIK_SIZES.items():
+    for name, s in design["sizes"]().items():
         if args.sizes and name not in args.sizes.split(","):
             continue
-        kav = KavuvikConfig(**kavuvik_config(s, n_layers, args.window))
-        llama = LlamaConfig(**closest_llama_config(s, n_layers))
-        print(f"[bench] {name}: Kavuvik", file=sys.stderr, flush=True)
-        k = measure(kav, lambda t, b=0, kv=0, s=s: kavuvik_work(s, n_layers, t, b, kv))
+        _, new = parse_config(design["config"](s, n_layers, args.window))
+        llama = LlamaConfig(**design["llama"](s, n_layers))
+        print(f"[bench] {name}: {label}", file=sys.stderr, flush=True)
+        k = measure(new, lambda t, b=0, kv=0, elt=2, s=s: design["work"](s, n_layers, t, b, kv, elt))
         print(f"[bench] {name}: Llama", file=sys.stderr, flush=True)
-        l = None if args.only_new else measure(llama, lambda t, b=0, kv=0, c=llama: llama_work(c, n_layers, t, b, kv))
-        sizes[name] = {"shape": s, "kavuvik": k, "llama": l}
-    first = sizes[next(iter(sizes))]["kavuvik"]["decode"]["batch8"]
+        l = None if args.only_new else measure(llama, lambda t, b=0, kv=0, elt=2, c=llama: llama_work(c, n_layers, t, b, kv))
+        sizes[name] = {"shape": s, args.workload: k, "llama": l}
+    first_name = next(iter(sizes))
+    first = sizes[first_name][args.workload]["decode"]["batch8"]
     return {
-        "metric": "decode tokens per second of Kavuvik layers (2048-wide, batch 8), beside Llama layers of equal size",
+        "metric": f"decode tokens per second of {label} layers ({first_name}, batch 8), beside Llama layers of equal size",
         "value": first["tok_per_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": first["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: seeded uniform-random token ids, random weights N(0, 0.02)",
-        "config": {"model": "Kavuvik and Llama layers", "layers": n_layers, "global_batch": 8, "seq_len": context,
+        "config": {"model": f"{label} and Llama layers", "layers": n_layers, "global_batch": 8, "seq_len": context,
                    "prefill_tokens": prompt, "window": args.window, "vocab_size": COMPARISON_VOCAB,
                    "hip_graph": not args.no_graph, "parallelism": "single GPU"},
         "sizes": sizes,
@@ -497,9 +576,9 @@ def main() -> int:
                          "by default (scheduling_steps_ahead); 0: read every step's tokens before the next is put together")
     ap.add_argument("--sampling", default="greedy", choices=["greedy", "temperature", "top_p", "top_k", "all"],
                     help="how the decode steps sample (the contract's line is greedy)")
-    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b", "kavuvik"],
+    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b", "kavuvik", "zabunex"],
                     help="decode8b: the headline line; mixed3b and llama70b run requests through the scheduler; "
-                         "kavuvik: prefill and decode of Kavuvik layers at two sizes beside the closest Llama layers")
+                         "kavuvik, zabunex: prefill and decode of that design's layers at two sizes beside the closest Llama layers")
     ap.add_argument("--sizes", default="", help="kavuvik: only these sizes (names with commas between them)")
     ap.add_argument("--only-new", action="store_true", help="kavuvik: leave the Llama layers out (for profiles)")
     ap.add_argument("--window", type=int, default=0,
@@ -511,7 +590,7 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
-    if args.workload == "kavuvik":
+    if args.workload in DESIGNS:
         print(json.dumps(design_comparison(args)), flush=True)
         return 0
     if args.workload != "decode8b":

@@ -190,7 +190,7 @@ int hal_clamped_gate_mul(const void* gu, void* out, int dtype, int n_tokens, int
                          float alpha, hipStream_t stream);
 
 // ---- rows of the stream and of projections (stream_ops.hip) -------------------------------
-// out = T(h), n elements (a multiple of 4)
+// out = T(h), n elements
 int hal_cast_rows(const float* h, void* out, int dtype, long long n, hipStream_t stream);
 // h[r] += a[r] * rsqrt(mean(a[r]^2) + eps) * w (float32 h and a, [n_rows, d]); cast (or
 // null) receives the new rows of h rounded to `dtype`.

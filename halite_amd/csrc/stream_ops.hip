@@ -21,11 +21,25 @@ __global__ void cast_rows_kernel(const float* __restrict__ h, T* __restrict__ ou
   load4(h + i * 4, v);
   store4(out + i * 4, v);
 }
+template <typename T>
+__global__ void cast_each_kernel(const float* __restrict__ h, T* __restrict__ out, long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = from_f32<T>(h[i]);
+}
 
 extern "C" int hal_cast_rows(const float* h, void* out, int dtype, long long n, hipStream_t stream) {
-  HAL_REQUIRE(n >= 0 && n % 4 == 0, "hal_cast_rows: %lld elements are not a multiple of 4", n);
+  HAL_REQUIRE(n >= 0, "hal_cast_rows: %lld elements", n);
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_cast_rows: dtype %d", dtype);
   if (n == 0) return 0;
+  if (n % 4 != 0 || ((uintptr_t)h % 16) != 0 || ((uintptr_t)out % 8) != 0) {  // no vectors of four
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == HAL_F32)
+      hipLaunchKernelGGL(cast_each_kernel<float>, dim3(blocks), dim3(256), 0, stream, h, (float*)out, n);
+    else
+      hipLaunchKernelGGL(cast_each_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, h, (bf16_t*)out, n);
+    HAL_LAUNCH_CHECK();
+    return 0;
+  }
   const long long n4 = n / 4;
   const unsigned blocks = (unsigned)((n4 + 255) / 256);
   if (dtype == HAL_F32)

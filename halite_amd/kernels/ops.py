@@ -860,7 +860,7 @@ def cast_rows(h: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
         return h
     lib = library.core_library()
     _dev(h)
-    _need(h.dtype == torch.float32 and h.numel() % 4 == 0, "cast_rows: float32 rows, a multiple of 4 elements")
+    _need(h.dtype == torch.float32, "cast_rows: float32 rows")
     out = torch.empty(h.shape, dtype=dtype, device=h.device)
     _check(lib, lib.hal_cast_rows(_ptr(h), _ptr(out), dtype_code(dtype), ctypes.c_longlong(h.numel()), _stream()))
     return out
