@@ -223,11 +223,15 @@ int hal_short_conv_carry(const float* u, int ldu, float* state, int taps, const 
                          const int* seg_q_len, const int* token_slot, int n_segs, int C,
                          hipStream_t stream);
 // xbc [T, ldx]: x (heads * P), then B and C (groups * N each).  state [slots][heads][N][P].
-// y [T, heads * P] float32 = S_t^T C_t + D x_t.
+// y [T, heads * P] float32 = S_t^T C_t + D x_t.  chunks [n_chunks][4] (first token, tokens,
+// segment, 0), seg_chunks [segments][2] (first chunk, chunks), sums (n_chunks * heads * N * P
+// floats) and decays (n_chunks * heads floats): the segments cut into chunks that are walked
+// side by side, or all null: a wave walks a whole segment.
 int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt_raw, int ld_dt,
                  const void* dt_bias, const void* a_log, const void* d_skip, int w_dtype,
                  float* state, const int* seg_q_start, const int* seg_q_len, const int* token_slot,
-                 float* y, int n_segs, int heads, int P, int N, int groups, hipStream_t stream);
+                 float* y, int n_segs, int heads, int P, int N, int groups, const int* chunks,
+                 const int* seg_chunks, int n_chunks, float* sums, float* decays, hipStream_t stream);
 // out = (y * silu(z)) / rms over each of `parts` equal parts of the row * w
 int hal_gated_part_norm(const float* y, const float* z, int ldz, const void* w, int w_dtype,
                         float eps, void* out, int dtype, int n_tokens, int inner, int parts,

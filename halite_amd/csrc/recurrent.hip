@@ -98,29 +98,42 @@ extern "C" int hal_short_conv_carry(const float* u, int ldu, float* state, int t
   return 0;
 }
 
-// ---- the recurrence: a wave takes 64 value channels of one head of one segment and walks
-// the segment's tokens; a lane holds its channel's column of the state (N numbers) in
-// registers, so the sums over the state need no exchange between lanes.  A token's B and C
-// (shared by the lanes) go through LDS, the next token's on their way meanwhile. ------------
-template <typename T, int NREG>
+// ---- the recurrence: a wave takes 64 value channels of one head of one run of tokens and
+// walks them; a lane holds its channel's column of the state (N numbers) in registers, so the
+// sums over the state need no exchange between lanes.  A token's B and C (shared by the
+// lanes) go through LDS, the next token's on their way meanwhile.
+//
+// MODE 0: a run is a segment; the state comes from the request's row and goes back there.
+// Long segments are cut into chunks (`chunks` [n][4]: first token, tokens, segment, unused),
+// so that the chip has a wave for every chunk and not for every request:
+// MODE 1: a run is a chunk, walked from a zero state; what it leaves (sums [chunk][head][N][P])
+//   and the product of its decays ([chunk][head]) are written, no output;
+// then a wave per (segment, head, 64 channels) takes the request's state through the
+//   segment's chunks in order, S <- decay_c S + sums_c, leaving in sums_c the state that
+//   chunk c starts from, and writes the last state to the request's row;
+// MODE 2: a run is a chunk again, walked from the state it starts from, for the outputs.
+// The result is the recurrence's own, token by token; only the order of additions differs. ----
+template <typename T, int NREG, int MODE>
 __global__ void __launch_bounds__(HAL_WAVE)
 ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt_raw, int ld_dt,
                 const void* __restrict__ dt_bias, const void* __restrict__ a_log, const void* __restrict__ d_skip,
                 int w_dtype, float* __restrict__ state, const int* __restrict__ seg_q_start,
                 const int* __restrict__ seg_q_len, const int* __restrict__ token_slot, float* __restrict__ y,
+                const int* __restrict__ chunks, float* __restrict__ sums, float* __restrict__ decays,
                 int heads, int P, int N, int groups) {
   __shared__ float bc[2][2 * NREG];
   const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int p = blockIdx.z * HAL_WAVE + lane;
-  const int t0 = seg_q_start[s], n = seg_q_len[s];
+  const int t0 = MODE == 0 ? seg_q_start[s] : chunks[s * 4], n = MODE == 0 ? seg_q_len[s] : chunks[s * 4 + 1];
   if (n <= 0) return;
   const int inner = heads * P;
   const int g = h / (heads / groups);
   const bool live = p < P;
-  float* st = state + (((size_t)token_slot[t0] * heads + h) * N) * P + (live ? p : 0);
+  float* st = MODE == 0 ? state + (((size_t)token_slot[t0] * heads + h) * N) * P + (live ? p : 0)
+                        : sums + (((size_t)s * heads + h) * N) * P + (live ? p : 0);
   float S[NREG];
 #pragma unroll
-  for (int i = 0; i < NREG; ++i) S[i] = (live && i < N) ? st[(size_t)i * P] : 0.f;
+  for (int i = 0; i < NREG; ++i) S[i] = (MODE != 1 && live && i < N) ? st[(size_t)i * P] : 0.f;
   const float rate = expf(load_as_f32(a_log, w_dtype, h));
   const float bias = load_as_f32(dt_bias, w_dtype, h);
   const float skip = load_as_f32(d_skip, w_dtype, h);
@@ -134,7 +147,7 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
     for (int u = 0; u < PER; ++u) {
       const int i = lane + u * HAL_WAVE;
       nb[u] = i < N ? to_f32(xbc[(size_t)t * ldx + b_col + i]) : 0.f;
-      nc[u] = i < N ? to_f32(xbc[(size_t)t * ldx + c_col + i]) : 0.f;
+      if (MODE != 1) nc[u] = i < N ? to_f32(xbc[(size_t)t * ldx + c_col + i]) : 0.f;
     }
   };
   auto put = [&](int buf) {
@@ -143,13 +156,14 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
       const int i = lane + u * HAL_WAVE;
       if (i < NREG) {
         bc[buf][i] = nb[u];
-        bc[buf][NREG + i] = nc[u];
+        if (MODE != 1) bc[buf][NREG + i] = nc[u];
       }
     }
   };
   ask(t0);
   float x_next = live ? to_f32(xbc[(size_t)t0 * ldx + (size_t)h * P + p]) : 0.f;
   float dt_next = dt_raw[(size_t)t0 * ld_dt + h];
+  float decay_all = 1.f;
   for (int i = 0; i < n; ++i) {
     const int t = t0 + i, buf = i & 1;
     put(buf);
@@ -165,52 +179,107 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
     const float dt = raw > 20.f ? raw : log1pf(expf(raw));
     const float decay = expf(-rate * dt);
     const float dtx = dt * x;
-    float acc0 = 0.f, acc1 = 0.f;
+    if (MODE == 1) {
+      decay_all *= decay;
 #pragma unroll
-    for (int k = 0; k < NREG; k += 2) {
-      S[k] = fmaf(decay, S[k], dtx * bc[buf][k]);
-      acc0 = fmaf(S[k], bc[buf][NREG + k], acc0);
-      S[k + 1] = fmaf(decay, S[k + 1], dtx * bc[buf][k + 1]);
-      acc1 = fmaf(S[k + 1], bc[buf][NREG + k + 1], acc1);
+      for (int k = 0; k < NREG; ++k) S[k] = fmaf(decay, S[k], dtx * bc[buf][k]);
+    } else {
+      float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+      for (int k = 0; k < NREG; k += 2) {
+        S[k] = fmaf(decay, S[k], dtx * bc[buf][k]);
+        acc0 = fmaf(S[k], bc[buf][NREG + k], acc0);
+        S[k + 1] = fmaf(decay, S[k + 1], dtx * bc[buf][k + 1]);
+        acc1 = fmaf(S[k + 1], bc[buf][NREG + k + 1], acc1);
+      }
+      if (live) y[(size_t)t * inner + (size_t)h * P + p] = (acc0 + acc1) + skip * x;
     }
-    if (live) y[(size_t)t * inner + (size_t)h * P + p] = (acc0 + acc1) + skip * x;
   }
-  if (live) {
+  if (MODE != 2 && live) {
 #pragma unroll
     for (int i = 0; i < NREG; ++i)
       if (i < N) st[(size_t)i * P] = S[i];
   }
+  if (MODE == 1 && blockIdx.z == 0 && lane == 0) decays[(size_t)s * heads + h] = decay_all;
 }
 
+// seg_chunks [segments][2]: a segment's first chunk and number of chunks
+template <int NREG>
+__global__ void __launch_bounds__(HAL_WAVE)
+ssd_carry_kernel(float* __restrict__ state, float* __restrict__ sums, const float* __restrict__ decays,
+                 const int* __restrict__ seg_chunks, const int* __restrict__ seg_q_start,
+                 const int* __restrict__ seg_q_len, const int* __restrict__ token_slot, int heads, int P, int N) {
+  const int s = blockIdx.x, h = blockIdx.y, p = blockIdx.z * HAL_WAVE + threadIdx.x;
+  if (seg_q_len[s] <= 0 || p >= P) return;
+  const int c0 = seg_chunks[s * 2], nc = seg_chunks[s * 2 + 1];
+  float* st = state + (((size_t)token_slot[seg_q_start[s]] * heads + h) * N) * P + p;
+  float S[NREG];
+#pragma unroll
+  for (int i = 0; i < NREG; ++i) S[i] = i < N ? st[(size_t)i * P] : 0.f;
+  for (int c = c0; c < c0 + nc; ++c) {
+    float* sm = sums + (((size_t)c * heads + h) * N) * P + p;
+    const float decay = decays[(size_t)c * heads + h];
+#pragma unroll
+    for (int i = 0; i < NREG; ++i) {
+      if (i < N) {
+        const float left = sm[(size_t)i * P];
+        sm[(size_t)i * P] = S[i];
+        S[i] = fmaf(decay, S[i], left);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NREG; ++i)
+    if (i < N) st[(size_t)i * P] = S[i];
+}
+
+// chunks, seg_chunks, sums, decays: all null (a wave walks a whole segment), or the cut of the
+// segments into n_chunks chunks and room for n_chunks * heads * N * P and n_chunks * heads floats.
 extern "C" int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt_raw, int ld_dt,
                             const void* dt_bias, const void* a_log, const void* d_skip, int w_dtype, float* state,
                             const int* seg_q_start, const int* seg_q_len, const int* token_slot, float* y,
-                            int n_segs, int heads, int P, int N, int groups, hipStream_t stream) {
+                            int n_segs, int heads, int P, int N, int groups, const int* chunks,
+                            const int* seg_chunks, int n_chunks, float* sums, float* decays, hipStream_t stream) {
   HAL_REQUIRE(n_segs >= 0 && heads > 0 && P > 0 && N > 0 && groups > 0 && heads % groups == 0,
               "hal_ssd_scan: bad sizes segments=%d heads=%d P=%d N=%d groups=%d", n_segs, heads, P, N, groups);
   HAL_REQUIRE(N <= 256, "hal_ssd_scan: a state of %d numbers a channel exceeds 256", N);
   HAL_REQUIRE(ldx >= heads * P + 2 * groups * N && ld_dt >= heads, "hal_ssd_scan: rows too short");
   HAL_REQUIRE(heads <= 65535 && (P + HAL_WAVE - 1) / HAL_WAVE <= 65535, "hal_ssd_scan: grid limit");
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_ssd_scan: dtype %d", dtype);
+  const bool cut = chunks != nullptr;
+  HAL_REQUIRE(!cut || (seg_chunks && sums && decays && n_chunks >= 0), "hal_ssd_scan: chunks without their buffers");
   if (n_segs == 0) return 0;
-  dim3 grid(n_segs, heads, (P + HAL_WAVE - 1) / HAL_WAVE);
-#define SCAN_LAUNCH(T_, N_)                                                                                  \
-  hipLaunchKernelGGL((ssd_scan_kernel<T_, N_>), grid, dim3(HAL_WAVE), 0, stream, (const T_*)xbc, ldx, dt_raw, \
-                     ld_dt, dt_bias, a_log, d_skip, w_dtype, state, seg_q_start, seg_q_len, token_slot, y,   \
-                     heads, P, N, groups)
-#define SCAN_BY_STATE(T_)                 \
-  do {                                    \
-    if (N <= 16) SCAN_LAUNCH(T_, 16);     \
-    else if (N <= 32) SCAN_LAUNCH(T_, 32);  \
-    else if (N <= 64) SCAN_LAUNCH(T_, 64);  \
-    else if (N <= 128) SCAN_LAUNCH(T_, 128); \
-    else SCAN_LAUNCH(T_, 256);            \
+  const dim3 block(HAL_WAVE);
+  const dim3 seg_grid(n_segs, heads, (P + HAL_WAVE - 1) / HAL_WAVE), chunk_grid(cut ? n_chunks : 1, heads, (P + HAL_WAVE - 1) / HAL_WAVE);
+#define SCAN_LAUNCH(T_, N_, MODE_, GRID_)                                                                      \
+  hipLaunchKernelGGL((ssd_scan_kernel<T_, N_, MODE_>), GRID_, block, 0, stream, (const T_*)xbc, ldx, dt_raw,    \
+                     ld_dt, dt_bias, a_log, d_skip, w_dtype, state, seg_q_start, seg_q_len, token_slot, y,     \
+                     chunks, sums, decays, heads, P, N, groups)
+#define SCAN_STEPS(T_, N_)                                                                                    \
+  do {                                                                                                        \
+    if (!cut) {                                                                                               \
+      SCAN_LAUNCH(T_, N_, 0, seg_grid);                                                                       \
+    } else if (n_chunks > 0) {                                                                                \
+      SCAN_LAUNCH(T_, N_, 1, chunk_grid);                                                                     \
+      hipLaunchKernelGGL((ssd_carry_kernel<N_>), seg_grid, block, 0, stream, state, sums, decays, seg_chunks, \
+                         seg_q_start, seg_q_len, token_slot, heads, P, N);                                    \
+      SCAN_LAUNCH(T_, N_, 2, chunk_grid);                                                                     \
+    }                                                                                                         \
+  } while (0)
+#define SCAN_BY_STATE(T_)                  \
+  do {                                     \
+    if (N <= 16) SCAN_STEPS(T_, 16);       \
+    else if (N <= 32) SCAN_STEPS(T_, 32);  \
+    else if (N <= 64) SCAN_STEPS(T_, 64);  \
+    else if (N <= 128) SCAN_STEPS(T_, 128); \
+    else SCAN_STEPS(T_, 256);              \
   } while (0)
   if (dtype == HAL_F32)
     SCAN_BY_STATE(float);
   else
     SCAN_BY_STATE(bf16_t);
 #undef SCAN_BY_STATE
+#undef SCAN_STEPS
 #undef SCAN_LAUNCH
   HAL_LAUNCH_CHECK();
   return 0;

@@ -173,6 +173,7 @@ class StepContext:
             tables[g.group_id] = bt
             pk.add(f"bt{g.group_id}", bt)
         self._packer = pk
+        self._shapes: dict = {}
         self._plans: dict = {}
         self._plan_host: dict = {}
         self._tables_host = tables
@@ -209,6 +210,27 @@ class StepContext:
             if self.static is not None:
                 raise RuntimeError("a static step needs its attention plans before the upload")
             self._plans[key] = attention_kernels.upload_plan(plan, self.device)
+
+    # A mixer's ``prepare`` may add int32 arrays of its own to the step's one copy, under a
+    # name; parts that ask for the same name share the array.
+    def add_array(self, name: str, make) -> None:
+        """``make()`` gives the int32 array ``name`` unless the step has it already; only
+        before the step's arrays go to the device."""
+        key = "part_" + name
+        if key in self._packer.offsets:
+            return
+        if self._dev is not None:
+            raise RuntimeError("a step's arrays are declared before its upload (in prepare)")
+        arr = np.ascontiguousarray(make(), dtype=np.int32)
+        self._shapes[key] = arr.shape
+        self._packer.add(key, arr)
+
+    def has_array(self, name: str) -> bool:
+        return "part_" + name in self._packer.offsets
+
+    def array(self, name: str) -> torch.Tensor:
+        key = "part_" + name
+        return self._view(key).view(self._shapes[key])
 
     def replace_tokens(self, tokens: np.ndarray) -> None:
         """Other token ids for a context that was put together before they were known

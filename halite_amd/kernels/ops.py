@@ -974,11 +974,15 @@ def short_conv_carry(u: torch.Tensor, state: torch.Tensor, seg_q_start: torch.Te
 
 def ssd_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor,
              d_skip: torch.Tensor, state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
-             token_slot: torch.Tensor, groups: int) -> torch.Tensor:
+             token_slot: torch.Tensor, groups: int, chunks: torch.Tensor | None = None,
+             seg_chunks: torch.Tensor | None = None) -> torch.Tensor:
     """The state-space recurrence over every request's tokens of the step.  ``xbc``
     ``[T, heads * P + 2 * groups * N]``: x, then B and C; ``dt_raw`` float32 ``[T, heads]``
     (a row-strided view is allowed); ``state`` float32 ``[slots, heads, N, P]``, read and
-    left as the step's last state.  Returns float32 ``[T, heads * P]``."""
+    left as the step's last state.  Returns float32 ``[T, heads * P]``.  ``chunks`` int32
+    ``[n, 4]`` (first token, tokens, segment, 0) and ``seg_chunks`` ``[segments, 2]`` (first
+    chunk, chunks): the segments cut into chunks that are walked side by side (what long
+    prompts need to fill the chip); without them a wave walks a whole segment."""
     lib = library.core_library()
     _dev(xbc, dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, token_slot)
     _, heads, n_state, p = state.shape
@@ -990,10 +994,21 @@ def ssd_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_l
     _need(dt_bias.numel() == heads and a_log.numel() == heads and d_skip.numel() == heads
           and dt_bias.dtype == a_log.dtype == d_skip.dtype, "ssd_scan: one bias, rate and skip a head, of one type")
     y = torch.empty((n, heads * p), dtype=torch.float32, device=xbc.device)
+    sums = decays = None
+    n_chunks = 0
+    if chunks is not None:
+        _dev(chunks, seg_chunks)
+        _i32(chunks, "chunks"), _i32(seg_chunks, "seg_chunks")
+        _need(chunks.dim() == 2 and chunks.shape[1] == 4 and seg_chunks is not None
+              and seg_chunks.shape == (seg_q_start.numel(), 2), "ssd_scan: chunk arrays")
+        n_chunks = chunks.shape[0]
+        sums = torch.empty((n_chunks, heads, n_state, p), dtype=torch.float32, device=xbc.device)
+        decays = torch.empty((n_chunks, heads), dtype=torch.float32, device=xbc.device)
     _check(lib, lib.hal_ssd_scan(
         _ptr(xbc), xbc.shape[1], dtype_code(xbc.dtype), _ptr(dt_raw), dt_raw.stride(0), _ptr(dt_bias), _ptr(a_log),
         _ptr(d_skip), dtype_code(a_log.dtype), _ptr(state), _ptr(seg_q_start), _ptr(seg_q_len), _ptr(token_slot),
-        _ptr(y), seg_q_start.numel(), heads, p, n_state, groups, _stream()))
+        _ptr(y), seg_q_start.numel(), heads, p, n_state, groups, _ptr(chunks), _ptr(seg_chunks), n_chunks,
+        _ptr(sums), _ptr(decays), _stream()))
     return y
 
 

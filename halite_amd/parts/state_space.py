@@ -12,11 +12,16 @@ inputs; it has no paged cache.  Decays, step sizes, state, gate and norm are flo
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 from pydantic import BaseModel, Field, StrictInt, model_validator
 
 from ..kernels import ops
 from .base import MIXERS, Mixer, ParamDecl, StateNeed
+
+
+# Tokens of a chunk of the recurrence where a step's longest segment has at least two of them.
+SCAN_CHUNK = 64
 
 
 class StateSpaceParams(BaseModel):
@@ -85,6 +90,25 @@ class StateSpace(Mixer):
             need["conv"] = StateNeed((p.conv_taps - 1, self.conv_channels))
         return need
 
+    def prepare(self, ctx, run):
+        # Long segments are cut into chunks that are walked side by side; the cut depends on
+        # the segments' token counts alone and is shared by every layer of the step.
+        lens = ctx.seg_q_len_host
+        if ctx.static is not None or len(lens) == 0 or int(lens.max()) < 2 * SCAN_CHUNK:
+            return
+        per_seg = -(-lens.astype(np.int64) // SCAN_CHUNK)
+        first = np.concatenate(([0], np.cumsum(per_seg)[:-1]))
+
+        def chunks():
+            seg = np.repeat(np.arange(len(lens)), per_seg)
+            k = np.arange(int(per_seg.sum())) - first[seg]
+            t0 = ctx.seg_q_start_host[seg] + k * SCAN_CHUNK
+            n = np.minimum(SCAN_CHUNK, lens[seg] - k * SCAN_CHUNK)
+            return np.stack((t0, n, seg, np.zeros_like(seg)), axis=1)
+
+        ctx.add_array(f"scan_chunks_{SCAN_CHUNK}", chunks)
+        ctx.add_array(f"scan_seg_chunks_{SCAN_CHUNK}", lambda: np.stack((first, per_seg), axis=1))
+
     def forward(self, x, ctx, run):
         p = self.p
         inner = self.inner
@@ -97,7 +121,10 @@ class StateSpace(Mixer):
                              ctx.token_slot, x.dtype, silu=True)
         if p.conv_taps > 1:
             ops.short_conv_carry(u, conv_state, ctx.seg_q_start, ctx.seg_q_len, ctx.token_slot)
+        cut = ctx.has_array(f"scan_chunks_{SCAN_CHUNK}")
         y = ops.ssd_scan(xbc, dt_raw, self.dt_bias, self.A_log, self.D, run.state["state"], ctx.seg_q_start,
-                         ctx.seg_q_len, ctx.token_slot, p.groups)
+                         ctx.seg_q_len, ctx.token_slot, p.groups,
+                         chunks=ctx.array(f"scan_chunks_{SCAN_CHUNK}") if cut else None,
+                         seg_chunks=ctx.array(f"scan_seg_chunks_{SCAN_CHUNK}") if cut else None)
         gated = ops.gated_part_norm(y, z, self.norm_weight, p.eps, p.norm_parts, x.dtype)
         return ops.linear(gated, self.out_weight, out_dtype=torch.float32, tiled=self.t_out)

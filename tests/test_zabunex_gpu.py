@@ -175,9 +175,11 @@ def test_short_convolution_in_steps(gpu, taps, act):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("shape", [(4, 16, 16, 2), (3, 8, 8, 1), (5, 12, 24, 5), (2, 80, 40, 2), (1, 64, 130, 1)])
-def test_state_space_recurrence_in_steps(gpu, dtype, shape):
+@pytest.mark.parametrize("chunk", [None, 3, 16])
+def test_state_space_recurrence_in_steps(gpu, dtype, shape, chunk):
     """The recurrence over two requests cut into steps against the whole sequences, the
-    state carried in float32 rows; decays from nearly 1 to nearly 0."""
+    state carried in float32 rows; decays from nearly 1 to nearly 0.  With ``chunk`` every
+    segment is cut into chunks of that many tokens that are walked side by side."""
     heads, Pd, N, G = shape
     T = {1: 37, 3: 12}
     x = {s: rand(n, heads * Pd + 2 * G * N, seed=20 + s).to(DT[dtype]) for s, n in T.items()}
@@ -197,7 +199,17 @@ def test_state_space_recurrence_in_steps(gpu, dtype, shape):
         xs = torch.cat([x[s][at[s] : at[s] + step[s]] for s in slots]).to(gpu)
         ds = torch.cat([dt[s][at[s] : at[s] + step[s]] for s in slots]).to(gpu)
         _, starts, lens, slot = step_arrays(gpu, cuts, slots)
-        y = ops.ssd_scan(xs, ds[:, 2:], dt_bias.to(gpu), a_log.to(gpu), skip.to(gpu), state, starts, lens, slot, G).cpu()
+        chunks = seg_chunks = None
+        if chunk:
+            rows, per_seg, t0 = [], [], 0
+            for i, n in enumerate(cuts):
+                per_seg.append((len(rows), -(-n // chunk)))
+                rows += [(t0 + k, min(chunk, n - k), i, 0) for k in range(0, n, chunk)]
+                t0 += n
+            chunks = torch.tensor(rows, dtype=torch.int32, device=gpu)
+            seg_chunks = torch.tensor(per_seg, dtype=torch.int32, device=gpu)
+        y = ops.ssd_scan(xs, ds[:, 2:], dt_bias.to(gpu), a_log.to(gpu), skip.to(gpu), state, starts, lens, slot, G,
+                         chunks=chunks, seg_chunks=seg_chunks).cpu()
         r = 0
         for s in slots:
             ref = want[s][at[s] : at[s] + step[s]].reshape(step[s], -1)
@@ -242,6 +254,31 @@ def test_schedules(folders, name, dtype, schedule):
     rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab"])
     check(rows, ref, dtype)
     assert runner.cache.idle()
+
+
+def test_long_prompts_whose_recurrence_is_cut_into_chunks(folders):
+    """Prompts of several chunks of the recurrence beside short ones in one step, against the
+    token-by-token model; then the same requests decoded on, so the carried state counts."""
+    from halite_amd.parts import state_space
+
+    for name, dtype in (("A", "float32"), ("B", "bfloat16")):
+        folder, _, _, weights = folders[(name, dtype)]
+        cfg = CONFIGS[name][0]
+        n = 4 * state_space.SCAN_CHUNK + 37
+        requests = {"long": tokens(cfg, n + 9, 61), "short": tokens(cfg, 5, 62), "mid": tokens(cfg, 2 * state_space.SCAN_CHUNK + 8, 63)}
+        ref = {rid: plain_logits(cfg, weights, ids) for rid, ids in requests.items()}
+        trace = [{"step": 0, "entries": [{"id": "long", "tokens": requests["long"][:n], "want": [0, n // 2, n - 1]},
+                                         {"id": "short", "tokens": requests["short"], "want": [4]},
+                                         {"id": "mid", "tokens": requests["mid"][:-3], "want": [100]}], "end": ["short"]}]
+        for i in range(n, n + 9):
+            entries = [{"id": "long", "tokens": [requests["long"][i]], "want": [0]}]
+            if i < n + 3:
+                entries.append({"id": "mid", "tokens": [requests["mid"][i - n - 3]], "want": [0]})
+            trace.append({"step": len(trace), "entries": entries, "end": ["mid"] if i == n + 2 else (["long"] if i == n + 8 else [])})
+        runner = make_runner(folder, dtype, replay.peak_tokens(trace, 16))
+        rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab"])
+        check(rows, ref, dtype)
+        assert runner.cache.idle()
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
