@@ -366,9 +366,9 @@ def llama_work(c, n_layers, tokens, batch=0, kv_tokens=0) -> dict:
 # mixer to every four, as many weights in the feed-forward's two matrices as in the three of
 # the Llama layer beside it (same width, heads, head size and grouping).
 ZABUNEX_SIZES = {
-    "2048-wide": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=12288, llama_ff=8192, chunk=1024, bias_max=2048,
+    "2048-wide": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=12288, llama_ff=8192, chunk=1024, bias_max=128,
                       ssm_heads=32, ssm_dim=64, state=128, groups=8),
-    "4096-wide": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=21504, llama_ff=14336, chunk=1024, bias_max=2048,
+    "4096-wide": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=21504, llama_ff=14336, chunk=1024, bias_max=128,
                       ssm_heads=64, ssm_dim=64, state=128, groups=8),
 }
 

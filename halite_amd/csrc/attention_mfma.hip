@@ -255,6 +255,16 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     m[rt] = -INFINITY;
     l[rt] = 0.f;
   }
+  // (RULED) what the table holds for every distance from its last one on: a step whose keys
+  // all lie that far behind the tile's first row needs no look-up by distance
+  float far_bias[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    far_bias[rt] = 0.f;
+    if constexpr (RULED) {
+      if (rule.bias) far_bias[rt] = rule.bias[(size_t)head[rt] * rule.bias_len + rule.bias_len - 1];
+    }
+  }
 
   const int last_key = kv_len - 1;  // keys beyond it are not written yet
   // page and slot of a key; pages of a power of two (page_shift >= 0) need no division
@@ -375,9 +385,11 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       const bool full = j0 >= kv_begin && j0 + KB <= kv_end && j0 + KB - 1 <= p_first[rt] &&
                         j0 >= lo_last[rt];
       // (RULED: sv holds scaled scores, in units of log2, with the bias added)
+      const bool far = RULED && p_first[rt] - (j0 + KB - 1) >= rule.bias_len - 1;  // (the same for the wave)
       auto ruled = [&](float raw, int j) {
         if constexpr (RULED) {
           if (rule.bias == nullptr) return raw * scale_log2e;
+          if (far) return __builtin_fmaf(raw, scale_log2e, far_bias[rt]);
           int back = p_row[rt] - j;
           back = back < 0 ? 0 : (back < rule.bias_len ? back : rule.bias_len - 1);
           return __builtin_fmaf(raw, scale_log2e, rule.bias[(size_t)head[rt] * rule.bias_len + back]);

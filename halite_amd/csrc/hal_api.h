@@ -192,10 +192,11 @@ int hal_clamped_gate_mul(const void* gu, void* out, int dtype, int n_tokens, int
 // ---- rows of the stream and of projections (stream_ops.hip) -------------------------------
 // out = T(h), n elements
 int hal_cast_rows(const float* h, void* out, int dtype, long long n, hipStream_t stream);
-// h[r] += a[r] * rsqrt(mean(a[r]^2) + eps) * w (float32 h and a, [n_rows, d]); cast (or
-// null) receives the new rows of h rounded to `dtype`.
-int hal_post_norm_add(float* h, const float* a, const void* w, int w_dtype, float eps, void* cast,
-                      int dtype, int n_rows, int d, hipStream_t stream);
+// h[r] += x * rsqrt(mean(x^2) + eps) * w with x = s1 * a[r] (+ s2 * a2[r] if a2 is given);
+// float32 h, a and a2, [n_rows, d]; cast (or null) receives the new rows of h rounded to `dtype`.
+int hal_post_norm_add(float* h, const float* a, const float* a2, float s1, float s2, const void* w,
+                      int w_dtype, float eps, void* cast, int dtype, int n_rows, int d,
+                      hipStream_t stream);
 int hal_relu_squared(const void* x, void* out, int dtype, long long n, hipStream_t stream);
 // y = alpha * y + beta * x
 int hal_scaled_sum_f32(float* y, float alpha, const float* x, float beta, long long n,

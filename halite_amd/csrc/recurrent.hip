@@ -121,7 +121,7 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
                 const int* __restrict__ seg_q_len, const int* __restrict__ token_slot, float* __restrict__ y,
                 const int* __restrict__ chunks, float* __restrict__ sums, float* __restrict__ decays,
                 int heads, int P, int N, int groups) {
-  __shared__ float bc[2][2 * NREG];
+  __shared__ __align__(16) float bc[2][2 * NREG];
   const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int p = blockIdx.z * HAL_WAVE + lane;
   const int t0 = MODE == 0 ? seg_q_start[s] : chunks[s * 4], n = MODE == 0 ? seg_q_len[s] : chunks[s * 4 + 1];
@@ -182,15 +182,27 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
     if (MODE == 1) {
       decay_all *= decay;
 #pragma unroll
-      for (int k = 0; k < NREG; ++k) S[k] = fmaf(decay, S[k], dtx * bc[buf][k]);
+      for (int k = 0; k < NREG; k += 4) {
+        const float4 b4 = *(const float4*)&bc[buf][k];
+        S[k] = fmaf(decay, S[k], dtx * b4.x);
+        S[k + 1] = fmaf(decay, S[k + 1], dtx * b4.y);
+        S[k + 2] = fmaf(decay, S[k + 2], dtx * b4.z);
+        S[k + 3] = fmaf(decay, S[k + 3], dtx * b4.w);
+      }
     } else {
       float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
-      for (int k = 0; k < NREG; k += 2) {
-        S[k] = fmaf(decay, S[k], dtx * bc[buf][k]);
-        acc0 = fmaf(S[k], bc[buf][NREG + k], acc0);
-        S[k + 1] = fmaf(decay, S[k + 1], dtx * bc[buf][k + 1]);
-        acc1 = fmaf(S[k + 1], bc[buf][NREG + k + 1], acc1);
+      for (int k = 0; k < NREG; k += 4) {
+        const float4 b4 = *(const float4*)&bc[buf][k];
+        const float4 c4 = *(const float4*)&bc[buf][NREG + k];
+        S[k] = fmaf(decay, S[k], dtx * b4.x);
+        acc0 = fmaf(S[k], c4.x, acc0);
+        S[k + 1] = fmaf(decay, S[k + 1], dtx * b4.y);
+        acc1 = fmaf(S[k + 1], c4.y, acc1);
+        S[k + 2] = fmaf(decay, S[k + 2], dtx * b4.z);
+        acc0 = fmaf(S[k + 2], c4.z, acc0);
+        S[k + 3] = fmaf(decay, S[k + 3], dtx * b4.w);
+        acc1 = fmaf(S[k + 3], c4.w, acc1);
       }
       if (live) y[(size_t)t * inner + (size_t)h * P + p] = (acc0 + acc1) + skip * x;
     }
@@ -203,34 +215,36 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
   if (MODE == 1 && blockIdx.z == 0 && lane == 0) decays[(size_t)s * heads + h] = decay_all;
 }
 
-// seg_chunks [segments][2]: a segment's first chunk and number of chunks
-template <int NREG>
-__global__ void __launch_bounds__(HAL_WAVE)
+// seg_chunks [segments][2]: a segment's first chunk and number of chunks.  A thread takes one
+// number of the state of one head of one segment through the segment's chunks; the chunks'
+// sums are asked for four at a time (the sums wait for each other, the loads need not).
+__global__ void __launch_bounds__(256)
 ssd_carry_kernel(float* __restrict__ state, float* __restrict__ sums, const float* __restrict__ decays,
                  const int* __restrict__ seg_chunks, const int* __restrict__ seg_q_start,
-                 const int* __restrict__ seg_q_len, const int* __restrict__ token_slot, int heads, int P, int N) {
-  const int s = blockIdx.x, h = blockIdx.y, p = blockIdx.z * HAL_WAVE + threadIdx.x;
-  if (seg_q_len[s] <= 0 || p >= P) return;
+                 const int* __restrict__ seg_q_len, const int* __restrict__ token_slot, int heads, int NP) {
+  const int s = blockIdx.x, h = blockIdx.y, e = blockIdx.z * blockDim.x + threadIdx.x;
+  if (seg_q_len[s] <= 0 || e >= NP) return;
   const int c0 = seg_chunks[s * 2], nc = seg_chunks[s * 2 + 1];
-  float* st = state + (((size_t)token_slot[seg_q_start[s]] * heads + h) * N) * P + p;
-  float S[NREG];
+  float* st = state + ((size_t)token_slot[seg_q_start[s]] * heads + h) * NP + e;
+  float S = *st;
+  constexpr int AHEAD = 4;
+  for (int c = c0; c < c0 + nc; c += AHEAD) {
+    float left[AHEAD], decay[AHEAD];
 #pragma unroll
-  for (int i = 0; i < NREG; ++i) S[i] = i < N ? st[(size_t)i * P] : 0.f;
-  for (int c = c0; c < c0 + nc; ++c) {
-    float* sm = sums + (((size_t)c * heads + h) * N) * P + p;
-    const float decay = decays[(size_t)c * heads + h];
+    for (int u = 0; u < AHEAD; ++u) {
+      const int cu = c + u < c0 + nc ? c + u : c0 + nc - 1;
+      left[u] = sums[((size_t)cu * heads + h) * NP + e];
+      decay[u] = decays[(size_t)cu * heads + h];
+    }
 #pragma unroll
-    for (int i = 0; i < NREG; ++i) {
-      if (i < N) {
-        const float left = sm[(size_t)i * P];
-        sm[(size_t)i * P] = S[i];
-        S[i] = fmaf(decay, S[i], left);
+    for (int u = 0; u < AHEAD; ++u) {
+      if (c + u < c0 + nc) {
+        sums[((size_t)(c + u) * heads + h) * NP + e] = S;
+        S = fmaf(decay[u], S, left[u]);
       }
     }
   }
-#pragma unroll
-  for (int i = 0; i < NREG; ++i)
-    if (i < N) st[(size_t)i * P] = S[i];
+  *st = S;
 }
 
 // chunks, seg_chunks, sums, decays: all null (a wave walks a whole segment), or the cut of the
@@ -250,6 +264,8 @@ extern "C" int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt
   HAL_REQUIRE(!cut || (seg_chunks && sums && decays && n_chunks >= 0), "hal_ssd_scan: chunks without their buffers");
   if (n_segs == 0) return 0;
   const dim3 block(HAL_WAVE);
+  HAL_REQUIRE(((long long)N * P + 255) / 256 <= 65535, "hal_ssd_scan: a state of %d x %d exceeds the grid limit", N, P);
+  const dim3 carry_grid(n_segs, heads, (N * P + 255) / 256);
   const dim3 seg_grid(n_segs, heads, (P + HAL_WAVE - 1) / HAL_WAVE), chunk_grid(cut ? n_chunks : 1, heads, (P + HAL_WAVE - 1) / HAL_WAVE);
 #define SCAN_LAUNCH(T_, N_, MODE_, GRID_)                                                                      \
   hipLaunchKernelGGL((ssd_scan_kernel<T_, N_, MODE_>), GRID_, block, 0, stream, (const T_*)xbc, ldx, dt_raw,    \
@@ -261,8 +277,8 @@ extern "C" int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt
       SCAN_LAUNCH(T_, N_, 0, seg_grid);                                                                       \
     } else if (n_chunks > 0) {                                                                                \
       SCAN_LAUNCH(T_, N_, 1, chunk_grid);                                                                     \
-      hipLaunchKernelGGL((ssd_carry_kernel<N_>), seg_grid, block, 0, stream, state, sums, decays, seg_chunks, \
-                         seg_q_start, seg_q_len, token_slot, heads, P, N);                                    \
+      hipLaunchKernelGGL(ssd_carry_kernel, carry_grid, dim3(256), 0, stream, state, sums, decays, seg_chunks, \
+                         seg_q_start, seg_q_len, token_slot, heads, N * P);                                   \
       SCAN_LAUNCH(T_, N_, 2, chunk_grid);                                                                     \
     }                                                                                                         \
   } while (0)

@@ -50,40 +50,45 @@ extern "C" int hal_cast_rows(const float* h, void* out, int dtype, long long n, 
   return 0;
 }
 
-// h[r] += a[r] * rsqrt(mean(a[r]^2) + eps) * w; cast (or null) receives the new row rounded to T
+// h[r] += x * rsqrt(mean(x^2) + eps) * w with x = s1 * a[r] (+ s2 * a2[r] if a2); cast (or
+// null) receives the new row rounded to T
 template <typename T>
 __global__ void post_norm_add_kernel(float* __restrict__ h, const float* __restrict__ a,
+                                     const float* __restrict__ a2, float s1, float s2,
                                      const void* __restrict__ w, int w_dtype, float eps,
                                      T* __restrict__ cast, int d) {
   __shared__ float scratch[16];
   const size_t r = blockIdx.x;
   const float* ar = a + r * d;
+  const float* br = a2 ? a2 + r * d : nullptr;
+  auto term = [&](int i) { return br ? __fadd_rn(__fmul_rn(s1, ar[i]), __fmul_rn(s2, br[i])) : __fmul_rn(s1, ar[i]); };
   float ss = 0.f;
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
-    const float x = ar[i];
+    const float x = term(i);
     ss += x * x;
   }
   const float total = block_sum(ss, scratch);
   const float rstd = 1.0f / sqrtf(total / (float)d + eps);
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
-    const float y = h[r * d + i] + ar[i] * rstd * load_as_f32(w, w_dtype, i);
+    const float y = h[r * d + i] + term(i) * rstd * load_as_f32(w, w_dtype, i);
     h[r * d + i] = y;
     if (cast) cast[r * d + i] = from_f32<T>(y);
   }
 }
 
-extern "C" int hal_post_norm_add(float* h, const float* a, const void* w, int w_dtype, float eps,
-                                 void* cast, int dtype, int n_rows, int d, hipStream_t stream) {
+extern "C" int hal_post_norm_add(float* h, const float* a, const float* a2, float s1, float s2, const void* w,
+                                 int w_dtype, float eps, void* cast, int dtype, int n_rows, int d,
+                                 hipStream_t stream) {
   HAL_REQUIRE(n_rows >= 0 && d > 0, "hal_post_norm_add: bad sizes rows=%d d=%d", n_rows, d);
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_post_norm_add: dtype %d", dtype);
   if (n_rows == 0) return 0;
   const int threads = d >= 1024 ? 256 : (d >= 256 ? 128 : 64);
   if (dtype == HAL_F32)
-    hipLaunchKernelGGL(post_norm_add_kernel<float>, dim3(n_rows), dim3(threads), 0, stream, h, a, w, w_dtype, eps,
-                       (float*)cast, d);
+    hipLaunchKernelGGL(post_norm_add_kernel<float>, dim3(n_rows), dim3(threads), 0, stream, h, a, a2, s1, s2, w,
+                       w_dtype, eps, (float*)cast, d);
   else
-    hipLaunchKernelGGL(post_norm_add_kernel<bf16_t>, dim3(n_rows), dim3(threads), 0, stream, h, a, w, w_dtype, eps,
-                       (bf16_t*)cast, d);
+    hipLaunchKernelGGL(post_norm_add_kernel<bf16_t>, dim3(n_rows), dim3(threads), 0, stream, h, a, a2, s1, s2, w,
+                       w_dtype, eps, (bf16_t*)cast, d);
   HAL_LAUNCH_CHECK();
   return 0;
 }
@@ -96,10 +101,33 @@ __global__ void relu_squared_kernel(const T* __restrict__ x, T* __restrict__ out
   out[i] = from_f32<T>(v * v);
 }
 
+template <typename T>
+__global__ void relu_squared_vec_kernel(const T* __restrict__ x, T* __restrict__ out, long long n4) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n4) return;
+  float v[4];
+  load4(x + i * 4, v);
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const float r = fmaxf(v[u], 0.f);
+    v[u] = r * r;
+  }
+  store4(out + i * 4, v);
+}
+
 extern "C" int hal_relu_squared(const void* x, void* out, int dtype, long long n, hipStream_t stream) {
   HAL_REQUIRE(n >= 0, "hal_relu_squared: %lld elements", n);
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_relu_squared: dtype %d", dtype);
   if (n == 0) return 0;
+  if (n % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+    const unsigned blocks = (unsigned)((n / 4 + 255) / 256);
+    if (dtype == HAL_F32)
+      hipLaunchKernelGGL(relu_squared_vec_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)x, (float*)out, n / 4);
+    else
+      hipLaunchKernelGGL(relu_squared_vec_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, (const bf16_t*)x, (bf16_t*)out, n / 4);
+    HAL_LAUNCH_CHECK();
+    return 0;
+  }
   const unsigned blocks = (unsigned)((n + 255) / 256);
   if (dtype == HAL_F32)
     hipLaunchKernelGGL(relu_squared_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)x, (float*)out, n);

@@ -867,18 +867,23 @@ def cast_rows(h: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 
 
 def post_norm_add(h: torch.Tensor, a: torch.Tensor, weight: torch.Tensor, eps: float,
-                  cast_to: torch.dtype | None = None):
-    """``h += a * rsqrt(mean(a^2) + eps) * weight`` row by row in float32 (``h`` and ``a``
-    float32 ``[T, d]``); with ``cast_to`` the new rows rounded to that type come back."""
+                  cast_to: torch.dtype | None = None, scale: float = 1.0, second: torch.Tensor | None = None,
+                  second_scale: float = 0.0):
+    """``h += x * rsqrt(mean(x^2) + eps) * weight`` row by row in float32 with
+    ``x = scale * a`` (``+ second_scale * second``: the sum of two parts' results); ``h``,
+    ``a`` and ``second`` float32 ``[T, d]``; with ``cast_to`` the new rows rounded to that
+    type come back."""
     lib = library.core_library()
-    _dev(h, a, weight)
+    _dev(h, a, weight, second)
     _need(h.dtype == torch.float32 and a.dtype == torch.float32 and h.dim() == 2 and a.shape == h.shape,
           "post_norm_add: float32 rows of one shape")
+    _need(second is None or (second.dtype == torch.float32 and second.shape == h.shape), "post_norm_add: the second term")
     _need(weight.shape == (h.shape[1],), "post_norm_add: weight of the rows' width")
     cast = None
     if cast_to is not None and cast_to != torch.float32:
         cast = torch.empty(h.shape, dtype=cast_to, device=h.device)
-    _check(lib, lib.hal_post_norm_add(_ptr(h), _ptr(a), _ptr(weight), dtype_code(weight.dtype), ctypes.c_float(eps),
+    _check(lib, lib.hal_post_norm_add(_ptr(h), _ptr(a), _ptr(second), ctypes.c_float(scale), ctypes.c_float(second_scale),
+                                      _ptr(weight), dtype_code(weight.dtype), ctypes.c_float(eps),
                                       _ptr(cast), dtype_code(cast_to or torch.float32), h.shape[0], h.shape[1], _stream()))
     return h if cast is None else cast
 

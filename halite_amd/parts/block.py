@@ -126,14 +126,35 @@ class PostNormBlock(Arrangement):
         if pending is not None:
             ops.residual_add(h, pending)
         dtype = self.mixer.build.dtype
-        a = self.mixer.forward(ops.cast_rows(h, dtype), ctx, run)
-        if a.dtype != torch.float32:
-            a = a.float()
-        x = ops.post_norm_add(h, a, self.mixer_norm.weight, self.mixer_norm.p.eps,
-                              cast_to=dtype if self.ff is not None else None)
-        if self.ff is not None:
+        # the rows as the block of the run before left them rounded, if that was one of this
+        # kind (then nothing has touched the stream since)
+        left = getattr(ctx, "rounded_rows", None)
+        ctx.rounded_rows = None
+        if pending is None and left is not None and left[0] == run.index - 1 and left[1].dtype == dtype and left[1].shape == h.shape:
+            x = left[1]
+        else:
+            x = ops.cast_rows(h, dtype)
+        norm = self.mixer_norm
+        last = self.ff is None
+        # a sum of two mixers is made by the kernel that norms it
+        terms = self.mixer.forward_terms(x, ctx, run) if hasattr(self.mixer, "forward_terms") else None
+        if terms is not None and len(terms) == 2:
+            (a, s1), (b, s2) = terms
+            x = ops.post_norm_add(h, a, norm.weight, norm.p.eps, cast_to=dtype, scale=s1, second=b, second_scale=s2)
+        else:
+            a = self.mixer.forward(x, ctx, run) if terms is None else None
+            if terms is not None:  # any other number of members: added up one by one
+                a = ops.scale_(terms[0][0], terms[0][1])
+                for b, s in terms[1:]:
+                    ops.scaled_sum_(a, 1.0, b, s)
+            if a.dtype != torch.float32:
+                a = a.float()
+            x = ops.post_norm_add(h, a, norm.weight, norm.p.eps, cast_to=dtype)
+        if not last:
             b = self.ff.forward(x, ctx)
             if b.dtype != torch.float32:
                 b = b.float()
-            ops.post_norm_add(h, b, self.ff_norm.weight, self.ff_norm.p.eps)
+            x = ops.post_norm_add(h, b, self.ff_norm.weight, self.ff_norm.p.eps, cast_to=dtype)
+        if dtype != torch.float32:
+            ctx.rounded_rows = (run.index, x)
         return None

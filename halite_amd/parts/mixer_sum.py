@@ -78,6 +78,15 @@ class MixerSum(Mixer):
         for name, m, _ in self.members:
             m.prepare(ctx, self._member_run(run, name))
 
+    def forward_terms(self, x, ctx, run):
+        """The members' results and their constants, for a caller that adds them up itself
+        (an arrangement whose next kernel reads the sum anyway)."""
+        terms = []
+        for name, m, scale in self.members:
+            a = m.forward(x, ctx, self._member_run(run, name))
+            terms.append((a if a.dtype == torch.float32 else a.float(), scale))
+        return terms
+
     def forward(self, x, ctx, run):
         total = None
         for name, m, scale in self.members:
