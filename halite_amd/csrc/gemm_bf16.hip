@@ -41,7 +41,7 @@ __device__ __forceinline__ bf16x8 load_frag(const bf16_t* p, bool valid) {
   return __builtin_bit_cast(bf16x8, raw);
 }
 
-enum { SK_OUT_BF16 = 0, SK_OUT_F32 = 1, SK_OUT_F32_ADD = 2 };
+enum { SK_OUT_BF16 = 0, SK_OUT_F32 = 1, SK_OUT_F32_ADD = 2, SK_OUT_BF16_RELU_SQUARED = 3 };
 
 // What the rotating epilogue needs beside the product.  Row r' = head * D + 16 * j + c of
 // the reordered weight is row head * D + 8 * j + c of the stored one for c < 8 and row
@@ -376,9 +376,12 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
     }
     if (GATED) v = v2 * (v / (1.0f + expf(-v)));  // set 0 is the gate, set 1 is up
     const size_t o = (size_t)m * ldc + n;
-    if (out_mode == SK_OUT_BF16)
+    if (out_mode == SK_OUT_BF16) {
       ((bf16_t*)C)[o] = f32_to_bf16(v);
-    else if (out_mode == SK_OUT_F32)
+    } else if (out_mode == SK_OUT_BF16_RELU_SQUARED) {
+      const float r = fmaxf(v, 0.f);
+      ((bf16_t*)C)[o] = f32_to_bf16(r * r);
+    } else if (out_mode == SK_OUT_F32)
       ((float*)C)[o] = v;
     else
       ((float*)C)[o] += v;
@@ -423,7 +426,8 @@ static int skinny_waves(int blocks, int steps) {
 }
 
 // X [M, K] bf16 (M <= 64), W [N, K] bf16, optional W2 [N, K] (gated form: W is the
-// gate's weight, W2 is up's).  out_mode: 0 bf16, 1 float32, 2 add into float32.
+// gate's weight, W2 is up's).  out_mode: 0 bf16, 1 float32, 2 add into float32, 3 the
+// square of relu of the result, as bf16.
 extern "C" int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const void* W2,
                                     int ldw, void* C, int ldc, int out_mode, int M, int N, int K,
                                     hipStream_t stream) {
@@ -432,7 +436,7 @@ extern "C" int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const
               K);
   HAL_REQUIRE(ldx >= K && (ldw >= K || ldw == 0) && ldc >= N && ldx % 8 == 0 && ldw % 8 == 0,
               "hal_gemm_bf16_skinny: leading dimensions %d %d %d", ldx, ldw, ldc);
-  HAL_REQUIRE(out_mode >= 0 && out_mode <= 2, "hal_gemm_bf16_skinny: out_mode %d", out_mode);
+  HAL_REQUIRE(out_mode >= 0 && out_mode <= 3, "hal_gemm_bf16_skinny: out_mode %d", out_mode);
   HAL_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)W2 % 16) == 0,
               "hal_gemm_bf16_skinny: operands must be 16-byte aligned");
   if (M == 0) return 0;

@@ -69,7 +69,7 @@ int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, float* C, int
                  int N, int K, hipStream_t stream);
 
 // X [M <= 64, K] bf16, W [N, K] bf16, optional W2 [N, K] (gated: up * silu(gate), W the gate).
-// out_mode: 0 bf16, 1 float32, 2 add into float32.
+// out_mode: 0 bf16, 1 float32, 2 add into float32, 3 bf16 of the square of relu of the result.
 int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const void* W2, int ldw, void* C,
                          int ldc, int out_mode, int M, int N, int K, hipStream_t stream);
 
@@ -206,10 +206,14 @@ int hal_scaled_sum_f32(float* y, float alpha, const float* x, float beta, long l
 // mean square of their whole row and multiplied by wq, wk; q further by
 // 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) if temp_every > 0; written as
 // packed rows [H heads | K key heads | K value heads] of D entries a head (the rest zero).
+// With k_pages (not null): keys and values are appended to the pages as well, as
+// hal_rope_append does it (for an attention that does not rotate).
 int hal_qk_norm_pack(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
                      const void* wq, const void* wk, int w_dtype, float eps, const int* positions,
                      float temp_coef, int temp_every, void* out, int row_stride, int dtype,
-                     int n_tokens, int H, int K, int dq, int dv, int D, hipStream_t stream);
+                     int n_tokens, int H, int K, int dq, int dv, int D, const int* token_seg,
+                     const int* block_table, int bt_stride, void* k_pages, void* v_pages,
+                     int page_size, int n_pages, int tiled, hipStream_t stream);
 
 // ---- mixers with a carried state (recurrent.hip) -----------------------------------------
 // y[t, c] = act(bias[c] + sum_j w[c, j] * u[t - taps + 1 + j, c]) over the tokens of each

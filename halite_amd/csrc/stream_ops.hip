@@ -159,9 +159,21 @@ __global__ void qk_norm_pack_kernel(const float* __restrict__ q, int ldq, const 
                                     const float* __restrict__ v, int ldv, const void* __restrict__ wq,
                                     const void* __restrict__ wk, int w_dtype, float eps,
                                     const int* __restrict__ positions, float temp_coef, int temp_every,
-                                    T* __restrict__ out, int row_stride, int H, int K, int dq, int dv, int D) {
+                                    T* __restrict__ out, int row_stride, int H, int K, int dq, int dv, int D,
+                                    const int* __restrict__ token_seg, const int* __restrict__ block_table,
+                                    int bt_stride, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                    int page_size, int n_pages, bool tiled) {
   __shared__ float scratch[16];
   const size_t t = blockIdx.x;
+  // with pages: keys and values go to the request's page of this position as well
+  long long page = -1;
+  int off = 0;
+  if (k_pages) {
+    const int pos = positions[t];
+    page = block_table[(size_t)token_seg[t] * bt_stride + pos / page_size];
+    off = pos % page_size;
+    if (page < 0 || page >= n_pages) page = -1;  // checked on the host
+  }
   const float* qr = q + t * ldq;
   const float* kr = k + t * ldk;
   const float* vr = v ? v + t * ldv : nullptr;
@@ -191,13 +203,21 @@ __global__ void qk_norm_pack_kernel(const float* __restrict__ q, int ldq, const 
     if (d < dv) y = vr ? vr[hd * dv + d] : kr[hd * dq + d];
     o[H * D + e] = from_f32<T>(x);
     o[(H + K) * D + e] = from_f32<T>(y);
+    if (page >= 0) {
+      k_pages[((size_t)page * K + hd) * page_size * D + kv_key_offset(tiled, page_size, D, off, d)] = from_f32<T>(x);
+      v_pages[((size_t)page * K + hd) * D * page_size + kv_value_offset(tiled, page_size, D, off, d)] = from_f32<T>(y);
+    }
   }
 }
 
 extern "C" int hal_qk_norm_pack(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
                                 const void* wq, const void* wk, int w_dtype, float eps, const int* positions,
                                 float temp_coef, int temp_every, void* out, int row_stride, int dtype,
-                                int n_tokens, int H, int K, int dq, int dv, int D, hipStream_t stream) {
+                                int n_tokens, int H, int K, int dq, int dv, int D, const int* token_seg,
+                                const int* block_table, int bt_stride, void* k_pages, void* v_pages,
+                                int page_size, int n_pages, int tiled, hipStream_t stream) {
+  HAL_REQUIRE(k_pages == nullptr || (v_pages && token_seg && block_table && positions && page_size > 0 && n_pages > 0),
+              "hal_qk_norm_pack: pages without the arrays that say where a token's key goes");
   HAL_REQUIRE(n_tokens >= 0 && H > 0 && K > 0 && dq > 0 && dv > 0 && D >= dq && D >= dv,
               "hal_qk_norm_pack: bad sizes T=%d H=%d K=%d dq=%d dv=%d D=%d", n_tokens, H, K, dq, dv, D);
   HAL_REQUIRE(v != nullptr || dv == dq, "hal_qk_norm_pack: values that are the keys have the keys' size");
@@ -207,10 +227,14 @@ extern "C" int hal_qk_norm_pack(const float* q, int ldq, const float* k, int ldk
   if (n_tokens == 0) return 0;
   if (dtype == HAL_F32)
     hipLaunchKernelGGL(qk_norm_pack_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, q, ldq, k, ldk, v, ldv, wq,
-                       wk, w_dtype, eps, positions, temp_coef, temp_every, (float*)out, row_stride, H, K, dq, dv, D);
+                       wk, w_dtype, eps, positions, temp_coef, temp_every, (float*)out, row_stride, H, K, dq, dv, D,
+                       token_seg, block_table, bt_stride, (float*)k_pages, (float*)v_pages, page_size, n_pages,
+                       tiled != 0);
   else
     hipLaunchKernelGGL(qk_norm_pack_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream, q, ldq, k, ldk, v, ldv, wq,
-                       wk, w_dtype, eps, positions, temp_coef, temp_every, (bf16_t*)out, row_stride, H, K, dq, dv, D);
+                       wk, w_dtype, eps, positions, temp_coef, temp_every, (bf16_t*)out, row_stride, H, K, dq, dv, D,
+                       token_seg, block_table, bt_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, n_pages,
+                       tiled != 0);
   HAL_LAUNCH_CHECK();
   return 0;
 }

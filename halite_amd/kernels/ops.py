@@ -512,9 +512,11 @@ def gemm_bf16_skinny(
     out_dtype: torch.dtype = torch.bfloat16,
     add_to: torch.Tensor | None = None,
     tiled_shape: tuple[int, int] | None = None,
+    relu_squared: bool = False,
 ):
     """``x @ w.T`` for at most 64 rows of bf16 ``x``; with ``w_up`` the gated form
-    ``(x @ w_up.T) * silu(x @ w.T)``; ``add_to`` (float32) receives ``+=``."""
+    ``(x @ w_up.T) * silu(x @ w.T)``; ``add_to`` (float32) receives ``+=``;
+    ``relu_squared``: the bf16 result is the square of relu of the product."""
     lib = library.core_library()
     _dev(x, add_to)
     _need(x.dtype == torch.bfloat16, "skinny gemm takes bf16")
@@ -542,6 +544,9 @@ def gemm_bf16_skinny(
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
         mode = 0 if out_dtype == torch.bfloat16 else 1
         _need(out_dtype in (torch.bfloat16, torch.float32), "skinny gemm: output dtype")
+    if relu_squared:
+        _need(mode == 0 and w_up is None, "skinny gemm: the square of relu goes with a plain bf16 result")
+        mode = 3
     _check(
         lib,
         lib.hal_gemm_bf16_skinny(
@@ -914,13 +919,17 @@ def _rows_f32(t: torch.Tensor, cols: int, what: str):
 def qk_norm_pack(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor | None, w_q: torch.Tensor, w_k: torch.Tensor,
                  eps: float, n_heads: int, n_kv_heads: int, qk_dim: int, v_dim: int, head_dim: int,
                  out_dtype: torch.dtype, positions: torch.Tensor | None = None, temp_coef: float = 0.0,
-                 temp_every: int = 0) -> torch.Tensor:
+                 temp_every: int = 0, token_seg: torch.Tensor | None = None, block_table: torch.Tensor | None = None,
+                 k_pages: torch.Tensor | None = None, v_pages: torch.Tensor | None = None, page_size: int = 0,
+                 tiled: bool = False) -> torch.Tensor:
     """From float32 projections (row-strided views allowed): ``q`` and ``k`` each divided by
     the root mean square of their whole row (all heads at once) and multiplied by their
     weights, ``q`` further by ``1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)`` at
     position ``p`` if ``temp_every`` > 0; the packed rows ``[q heads | k heads | v heads]``
     of ``head_dim`` entries a head (zero beyond ``qk_dim`` / ``v_dim``) come back.  ``v``
-    None: the values are the keys as they were projected."""
+    None: the values are the keys as they were projected.  With ``k_pages`` and ``v_pages``
+    keys and values are appended to the pages as well, as ``rope_append`` does it (for an
+    attention that does not rotate)."""
     lib = library.core_library()
     n = q.shape[0]
     _rows_f32(q, n_heads * qk_dim, "qk_norm_pack q"), _rows_f32(k, n_kv_heads * qk_dim, "qk_norm_pack k")
@@ -933,10 +942,22 @@ def qk_norm_pack(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor | None, w_q: 
     _need(head_dim >= max(qk_dim, v_dim) and (v is not None or v_dim == qk_dim), "qk_norm_pack: head sizes")
     _need(temp_every == 0 or (positions is not None and positions.numel() == n), "qk_norm_pack: positions")
     out = torch.empty((n, (n_heads + 2 * n_kv_heads) * head_dim), dtype=out_dtype, device=q.device)
+    n_pages = 0
+    if k_pages is not None:
+        _dev(token_seg, block_table, k_pages, v_pages)
+        _i32(token_seg, "token_seg"), _i32(block_table, "block_table")
+        n_pages = k_pages.shape[0]
+        _need(v_pages is not None and k_pages.dtype == out_dtype and v_pages.dtype == out_dtype
+              and k_pages.shape == (n_pages, n_kv_heads, page_size, head_dim)
+              and v_pages.shape == (n_pages, n_kv_heads, head_dim, page_size), "qk_norm_pack: page shapes")
+        _need(positions is not None and positions.numel() == n and token_seg is not None and token_seg.numel() == n
+              and block_table is not None and block_table.dim() == 2, "qk_norm_pack: the step's arrays")
     _check(lib, lib.hal_qk_norm_pack(
         _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), 0 if v is None else v.stride(0), _ptr(w_q), _ptr(w_k),
         dtype_code(w_q.dtype), ctypes.c_float(eps), _ptr(positions), ctypes.c_float(temp_coef), temp_every,
-        _ptr(out), out.shape[1], dtype_code(out_dtype), n, n_heads, n_kv_heads, qk_dim, v_dim, head_dim, _stream()))
+        _ptr(out), out.shape[1], dtype_code(out_dtype), n, n_heads, n_kv_heads, qk_dim, v_dim, head_dim,
+        _ptr(token_seg), _ptr(block_table), 0 if block_table is None else block_table.shape[1],
+        _ptr(k_pages), _ptr(v_pages), page_size, n_pages, 1 if tiled else 0, _stream()))
     return out
 
 

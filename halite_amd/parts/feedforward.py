@@ -127,5 +127,10 @@ class DenseFeedForward(FeedForward):
                 self.t_out = ops.tile_weight(self.linear_out_weight)
 
     def forward(self, x, ctx, then=None):
-        act = ops.relu_squared(ops.linear(x, self.linear_up_weight, tiled=self.t_up))
+        m, d = x.shape
+        if self.t_up is not None and x.dtype == torch.bfloat16 and m <= ops.SKINNY_ROWS and d % 8 == 0:
+            # few rows: the activation is the product's epilogue
+            act = ops.gemm_bf16_skinny(x, self.t_up, tiled_shape=tuple(self.linear_up_weight.shape), relu_squared=True)
+        else:
+            act = ops.relu_squared(ops.linear(x, self.linear_up_weight, tiled=self.t_up))
         return ops.linear(act, self.linear_out_weight, out_dtype=torch.float32, tiled=self.t_out)

@@ -209,21 +209,19 @@ class NormedAttention(Mixer):
         q, k = a[:, : self.n_q], a[:, self.n_q : self.n_q + self.n_k]
         v = None if p.values_from_keys else a[:, self.n_q + self.n_k :]
         temp = p.q_temperature
+        # without a rotation the kernel that norms and packs appends to the pages itself
+        appends_here = self.position is None and run.appends
+        pages = dict(token_seg=ctx.token_seg, block_table=group.block_table, k_pages=kv.k, v_pages=kv.v,
+                     page_size=group.page_size, tiled=kv.tiled)
         packed = ops.qk_norm_pack(
             q, k, v, self.w_q_norm, self.w_k_norm, p.eps, p.n_heads, p.n_kv_heads, p.qk_dim, p.v_dim, D, x.dtype,
             positions=ctx.positions, temp_coef=temp.coef if temp else 0.0, temp_every=temp.every if temp else 0,
+            **(pages if appends_here else {}),
         )
         if self.position is not None:
             cos, sin = self.position.tables(ctx.max_position + 1)
-            rot, interleaved = self.position.rotary_dim, self.position.interleaved
-        else:
-            cos = sin = ctx.empty_f32
-            rot, interleaved = 0, False
-        ops.rope_append(
-            packed, ctx.positions, cos, sin, p.n_heads, p.n_kv_heads if run.appends else 0, D, rot, interleaved,
-            token_seg=ctx.token_seg, block_table=group.block_table,
-            k_pages=kv.k, v_pages=kv.v, page_size=group.page_size, tiled=kv.tiled,
-        )
+            ops.rope_append(packed, ctx.positions, cos, sin, p.n_heads, p.n_kv_heads if run.appends else 0, D,
+                            self.position.rotary_dim, self.position.interleaved, **pages)
         out = ctx.attention(packed, packed.shape[1], kv, group, p.n_heads, p.scale, p.window or 0, rule=self.rule)
         if D != p.v_dim:
             heads = torch.empty((n, p.n_heads * p.v_dim), dtype=out.dtype, device=out.device)

@@ -106,6 +106,11 @@ def test_square_of_relu_and_scaled_sum(gpu, dtype):
     x = rand(33, 50, seed=4).to(DT[dtype])
     got = ops.relu_squared(x.to(gpu)).float().cpu()
     assert float((got - P.relu_squared(x.float()).to(DT[dtype]).float()).abs().max()) == 0.0
+    if dtype == "bfloat16":  # few rows: the activation as the product's epilogue
+        a, w = rand(5, 64, seed=14).to(DT[dtype]), rand(48, 64, seed=15, scale=0.3).to(DT[dtype])
+        got = ops.gemm_bf16_skinny(a.to(gpu), ops.tile_weight(w.to(gpu)), tiled_shape=(48, 64), relu_squared=True).float().cpu()
+        want = P.relu_squared(a.float() @ w.float().T)
+        assert float((got - want).abs().max()) < 2e-2 * float(want.abs().max())
     y, z = rand(7, 12, seed=5), rand(7, 12, seed=6)
     got = ops.scaled_sum_(y.to(gpu), 0.6, z.to(gpu), -1.1).cpu()
     assert float((got - (0.6 * y - 1.1 * z)).abs().max()) < 1e-6
