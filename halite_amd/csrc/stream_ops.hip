@@ -76,12 +76,75 @@ __global__ void post_norm_add_kernel(float* __restrict__ h, const float* __restr
   }
 }
 
+// The same for rows of a multiple of four elements, up to 4 * VMAX * threads: a thread keeps
+// its part of the row in registers between the sum of squares and the update, and every
+// access is 16 bytes (a few rows of a decode step are a few workgroups whose time is the
+// chain of their trips to memory).
+template <typename T, int VMAX>
+__global__ void post_norm_add_vec_kernel(float* __restrict__ h, const float* __restrict__ a,
+                                         const float* __restrict__ a2, float s1, float s2,
+                                         const void* __restrict__ w, int w_dtype, float eps,
+                                         T* __restrict__ cast, int d) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  const int nv = d / 4;
+  float x[VMAX][4], hv[VMAX][4], wv[VMAX][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < VMAX; ++u) {
+    const int v = threadIdx.x + u * blockDim.x;
+    if (v < nv) {
+      load4(a + r * d + v * 4, x[u]);
+      load4(h + r * d + v * 4, hv[u]);
+      load4_any(w, w_dtype, (size_t)v * 4, wv[u]);
+      if (a2) {
+        float y[4];
+        load4(a2 + r * d + v * 4, y);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[u][i] = __fadd_rn(__fmul_rn(s1, x[u][i]), __fmul_rn(s2, y[i]));
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[u][i] = __fmul_rn(s1, x[u][i]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ss += x[u][i] * x[u][i];
+    }
+  }
+  const float total = block_sum(ss, scratch);
+  const float rstd = 1.0f / sqrtf(total / (float)d + eps);
+#pragma unroll
+  for (int u = 0; u < VMAX; ++u) {
+    const int v = threadIdx.x + u * blockDim.x;
+    if (v < nv) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) hv[u][i] = hv[u][i] + x[u][i] * rstd * wv[u][i];
+      store4(h + r * d + v * 4, hv[u]);
+      if (cast) store4(cast + r * d + v * 4, hv[u]);
+    }
+  }
+}
+
 extern "C" int hal_post_norm_add(float* h, const float* a, const float* a2, float s1, float s2, const void* w,
                                  int w_dtype, float eps, void* cast, int dtype, int n_rows, int d,
                                  hipStream_t stream) {
   HAL_REQUIRE(n_rows >= 0 && d > 0, "hal_post_norm_add: bad sizes rows=%d d=%d", n_rows, d);
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_post_norm_add: dtype %d", dtype);
   if (n_rows == 0) return 0;
+  constexpr int VMAX = 8;
+  const bool aligned = d % 4 == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)a2 % 16) == 0 &&
+                       ((uintptr_t)w % 16) == 0 && ((uintptr_t)cast % 16) == 0;
+  if (aligned && d <= 4 * VMAX * 256) {
+    const int nv = d / 4;
+    const int threads = nv >= 1024 ? 256 : (nv >= 256 ? 128 : 64);  // (at most VMAX vectors a thread)
+    if (dtype == HAL_F32)
+      hipLaunchKernelGGL((post_norm_add_vec_kernel<float, VMAX>), dim3(n_rows), dim3(threads), 0, stream, h, a, a2, s1,
+                         s2, w, w_dtype, eps, (float*)cast, d);
+    else
+      hipLaunchKernelGGL((post_norm_add_vec_kernel<bf16_t, VMAX>), dim3(n_rows), dim3(threads), 0, stream, h, a, a2, s1,
+                         s2, w, w_dtype, eps, (bf16_t*)cast, d);
+    HAL_LAUNCH_CHECK();
+    return 0;
+  }
   const int threads = d >= 1024 ? 256 : (d >= 256 ? 128 : 64);
   if (dtype == HAL_F32)
     hipLaunchKernelGGL(post_norm_add_kernel<float>, dim3(n_rows), dim3(threads), 0, stream, h, a, a2, s1, s2, w,
@@ -210,6 +273,91 @@ __global__ void qk_norm_pack_kernel(const float* __restrict__ q, int ldq, const 
   }
 }
 
+// The same with 16-byte accesses, for head sizes, row lengths and addresses in steps of four.
+template <typename T>
+__global__ void qk_norm_pack_vec_kernel(const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk,
+                                        const float* __restrict__ v, int ldv, const void* __restrict__ wq,
+                                        const void* __restrict__ wk, int w_dtype, float eps,
+                                        const int* __restrict__ positions, float temp_coef, int temp_every,
+                                        T* __restrict__ out, int row_stride, int H, int K, int dq, int dv, int D,
+                                        const int* __restrict__ token_seg, const int* __restrict__ block_table,
+                                        int bt_stride, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                        int page_size, int n_pages, bool tiled) {
+  __shared__ float scratch[16];
+  const size_t t = blockIdx.x;
+  long long page = -1;
+  int off = 0;
+  if (k_pages) {
+    const int pos = positions[t];
+    page = block_table[(size_t)token_seg[t] * bt_stride + pos / page_size];
+    off = pos % page_size;
+    if (page < 0 || page >= n_pages) page = -1;  // checked on the host
+  }
+  const float* qr = q + t * ldq;
+  const float* kr = k + t * ldk;
+  const float* vr = v ? v + t * ldv : nullptr;
+  const int nq = H * dq, nk = K * dq;
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x * 4; i < nq; i += blockDim.x * 4) {
+    float x[4];
+    load4(qr + i, x);
+    sq += (x[0] * x[0] + x[1] * x[1]) + (x[2] * x[2] + x[3] * x[3]);
+  }
+  for (int i = threadIdx.x * 4; i < nk; i += blockDim.x * 4) {
+    float x[4];
+    load4(kr + i, x);
+    sk += (x[0] * x[0] + x[1] * x[1]) + (x[2] * x[2] + x[3] * x[3]);
+  }
+  const float tq = block_sum(sq, scratch);
+  const float tk = block_sum(sk, scratch);
+  float rq = 1.0f / sqrtf(tq / (float)nq + eps);
+  const float rk = 1.0f / sqrtf(tk / (float)nk + eps);
+  if (temp_every > 0) {
+    const int p = positions[t];
+    rq *= 1.0f + temp_coef * logf((float)((p + 1) / temp_every + 1));
+  }
+  T* o = out + t * row_stride;
+  const int D4 = D / 4;
+  for (int e = threadIdx.x; e < H * D4; e += blockDim.x) {
+    const int hd = e / D4, d = (e % D4) * 4;
+    float x[4] = {0.f, 0.f, 0.f, 0.f};
+    if (d < dq) {
+      float wv[4];
+      load4(qr + hd * dq + d, x);
+      load4_any(wq, w_dtype, (size_t)hd * dq + d, wv);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] = x[i] * rq * wv[i];
+    }
+    store4(o + (size_t)hd * D + d, x);
+  }
+  for (int e = threadIdx.x; e < K * D4; e += blockDim.x) {
+    const int hd = e / D4, d = (e % D4) * 4;
+    float x[4] = {0.f, 0.f, 0.f, 0.f}, y[4] = {0.f, 0.f, 0.f, 0.f}, raw[4] = {0.f, 0.f, 0.f, 0.f};
+    if (d < dq) {
+      float wv[4];
+      load4(kr + hd * dq + d, raw);
+      load4_any(wk, w_dtype, (size_t)hd * dq + d, wv);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] = raw[i] * rk * wv[i];
+    }
+    if (d < dv) {
+      if (vr) load4(vr + hd * dv + d, y);
+      else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) y[i] = raw[i];
+      }
+    }
+    store4(o + (size_t)(H + hd) * D + d, x);
+    store4(o + (size_t)(H + K + hd) * D + d, y);
+    if (page >= 0) {
+      store4(k_pages + ((size_t)page * K + hd) * page_size * D + kv_key_offset(tiled, page_size, D, off, d), x);
+      T* vp = v_pages + ((size_t)page * K + hd) * D * page_size;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) vp[kv_value_offset(tiled, page_size, D, off, d + i)] = from_f32<T>(y[i]);
+    }
+  }
+}
+
 extern "C" int hal_qk_norm_pack(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
                                 const void* wq, const void* wk, int w_dtype, float eps, const int* positions,
                                 float temp_coef, int temp_every, void* out, int row_stride, int dtype,
@@ -225,6 +373,24 @@ extern "C" int hal_qk_norm_pack(const float* q, int ldq, const float* k, int ldk
   HAL_REQUIRE(temp_every == 0 || positions != nullptr, "hal_qk_norm_pack: a temperature needs positions");
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_qk_norm_pack: dtype %d", dtype);
   if (n_tokens == 0) return 0;
+  const bool by_four = dq % 4 == 0 && dv % 4 == 0 && D % 4 == 0 && ldq % 4 == 0 && ldk % 4 == 0 && ldv % 4 == 0 &&
+                       row_stride % 4 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 &&
+                       ((uintptr_t)v % 16) == 0 && ((uintptr_t)wq % 16) == 0 && ((uintptr_t)wk % 16) == 0 &&
+                       ((uintptr_t)out % 16) == 0 && ((uintptr_t)k_pages % 16) == 0;
+  if (by_four) {
+    if (dtype == HAL_F32)
+      hipLaunchKernelGGL(qk_norm_pack_vec_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, q, ldq, k, ldk, v, ldv,
+                         wq, wk, w_dtype, eps, positions, temp_coef, temp_every, (float*)out, row_stride, H, K, dq, dv,
+                         D, token_seg, block_table, bt_stride, (float*)k_pages, (float*)v_pages, page_size, n_pages,
+                         tiled != 0);
+    else
+      hipLaunchKernelGGL(qk_norm_pack_vec_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream, q, ldq, k, ldk, v, ldv,
+                         wq, wk, w_dtype, eps, positions, temp_coef, temp_every, (bf16_t*)out, row_stride, H, K, dq, dv,
+                         D, token_seg, block_table, bt_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, n_pages,
+                         tiled != 0);
+    HAL_LAUNCH_CHECK();
+    return 0;
+  }
   if (dtype == HAL_F32)
     hipLaunchKernelGGL(qk_norm_pack_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, q, ldq, k, ldk, v, ldv, wq,
                        wk, w_dtype, eps, positions, temp_coef, temp_every, (float*)out, row_stride, H, K, dq, dv, D,

@@ -89,12 +89,20 @@ def step_arrays(gpu, cuts, slots):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("sizes", [(1, 40), (37, 64), (5, 1028)])
-def test_norm_of_a_result_added_to_the_stream(gpu, dtype, sizes):
+@pytest.mark.parametrize("sizes", [(1, 40), (37, 64), (5, 1028), (3, 4096), (2, 8200), (4, 30)])
+@pytest.mark.parametrize("two", [False, True])
+def test_norm_of_a_result_added_to_the_stream(gpu, dtype, sizes, two):
+    """Rows of a few vectors a thread, of more than a thread keeps, and of a length that is
+    no multiple of four; one result, or the sum of two with a constant each."""
     t, d = sizes
     h, a, w = rand(t, d, seed=1), rand(t, d, seed=2, scale=3.0), (1 + 0.2 * rand(d, seed=3)).to(DT[dtype])
+    b = rand(t, d, seed=4, scale=2.0)
     hg = h.to(gpu)
-    cast = ops.post_norm_add(hg, a.to(gpu), w.to(gpu), 1e-5, cast_to=DT[dtype])
+    if two:
+        cast = ops.post_norm_add(hg, a.to(gpu), w.to(gpu), 1e-5, cast_to=DT[dtype], scale=0.6, second=b.to(gpu), second_scale=-1.1)
+        a = 0.6 * a.to(F) - 1.1 * b.to(F)
+    else:
+        cast = ops.post_norm_add(hg, a.to(gpu), w.to(gpu), 1e-5, cast_to=DT[dtype])
     want = h.to(F) + P.rms_norm(a.to(F), w.to(F), 1e-5)
     assert float((hg.cpu() - want).abs().max()) < 2e-6 * float(want.abs().max())
     assert torch.equal(cast.float().cpu(), hg.cpu().to(DT[dtype]).float())
@@ -117,20 +125,23 @@ def test_square_of_relu_and_scaled_sum(gpu, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", [(3, 1, 20, 20, 32, True), (4, 2, 16, 16, 16, True), (2, 1, 24, 8, 32, False), (5, 5, 4, 12, 16, False)])
-def test_whole_projection_norms_and_packed_rows(gpu, dtype, shape):
+@pytest.mark.parametrize("shape", [(3, 1, 20, 20, 32, True), (4, 2, 16, 16, 16, True), (2, 1, 24, 8, 32, False), (5, 5, 4, 12, 16, False),
+                                   (3, 3, 6, 10, 16, False)])
+@pytest.mark.parametrize("first", [5, 8])
+def test_whole_projection_norms_and_packed_rows(gpu, dtype, shape, first):
     """q and k over all heads at once, the temperature by position, the values the raw keys or
-    a projection of their own; heads padded to the pages' head size."""
+    a projection of their own; heads padded to the pages' head size.  Rows that begin at a
+    multiple of four columns (16-byte accesses) and rows that do not."""
     H, K, dq, dv, D, from_keys = shape
     t = 29
-    a = rand(t, 5 + H * dq + K * dq + K * dv, seed=7, scale=2.0)
-    q, k = a[:, 5 : 5 + H * dq], a[:, 5 + H * dq : 5 + (H + K) * dq]
-    v = None if from_keys else a[:, 5 + (H + K) * dq :]
+    a = rand(t, 8 + H * dq + K * dq + K * dv, seed=7, scale=2.0)[:, 8 - first :]
+    q, k = a[:, first : first + H * dq], a[:, first + H * dq : first + (H + K) * dq]
+    v = None if from_keys else a[:, first + (H + K) * dq :]
     wq, wk = (1 + 0.3 * rand(H * dq, seed=8)).to(DT[dtype]), (1 + 0.3 * rand(K * dq, seed=9)).to(DT[dtype])
     pos = torch.arange(t, dtype=torch.int32) * 3 + 1
-    ag = a.to(gpu)
+    ag = a.contiguous().to(gpu)
     packed = ops.qk_norm_pack(
-        ag[:, 5 : 5 + H * dq], ag[:, 5 + H * dq : 5 + (H + K) * dq], None if from_keys else ag[:, 5 + (H + K) * dq :],
+        ag[:, first : first + H * dq], ag[:, first + H * dq : first + (H + K) * dq], None if from_keys else ag[:, first + (H + K) * dq :],
         wq.to(gpu), wk.to(gpu), 1e-5, H, K, dq, dv, D, DT[dtype], positions=pos.to(gpu), temp_coef=0.4, temp_every=4,
     ).float().cpu().view(t, H + 2 * K, D)
     temp = 1 + 0.4 * torch.log((torch.div(pos + 1, 4, rounding_mode="floor") + 1).to(F))
