@@ -381,11 +381,11 @@ def zabunex_config(s, n_layers, window):
     attention = dict(heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["dim"], scale=s["dim"] ** -0.5,
                      bias_max=s["bias_max"], bias_buckets=32, q_temp=dict(coef=0.1, every=1024))
     left = dict(heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["dim"], scale=s["dim"] ** -0.5, conv=4,
-                mask=dict(size=s["chunk"]), rot=dict(base=500000.0, dims=64, scaling=dict(factor=8.0)))
+                mask=dict(size=s["chunk"]), rot=dict(base=500000.0, dims=64, scaling=dict(factor=4.0)))
     right = dict(heads=s["ssm_heads"], vdim=s["ssm_dim"], state=s["state"], groups=s["groups"], conv=4, norm_groups=s["groups"])
     mlp = dict(kind="dense", ff=s["ff"])
     layers = [dict(type="attention", mixer=attention, mlp=mlp) if kind == "attention" else
-              dict(type="parallel", mixer=dict(left=left, right=right, left_scale=0.6, right_scale=1.1), mlp=mlp)
+              dict(type="parallel", mixer=dict(left=left, right=right, left_scale=0.5, right_scale=1.0), mlp=mlp)
               for kind in zabunex_layer_kinds(n_layers)]
     return dict(architecture="Zabunex", vocab=COMPARISON_VOCAB, width=s["width"], norm=dict(eps=1e-5), max_positions=8192,
                 layers=layers)

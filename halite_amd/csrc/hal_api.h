@@ -223,6 +223,11 @@ int hal_short_conv(const float* u, int ldu, const void* w, const void* bias, int
                    const float* state, const int* token_seg, const int* seg_q_start,
                    const int* token_slot, void* y, int ldy, int y_dtype, int act, int n_tokens,
                    int C, hipStream_t stream);
+// Both in one kernel for a step in which every request brings one token (token t belongs to
+// slot token_slot[t], no two tokens to the same): y as above, and the state moved one on.
+int hal_short_conv_step(const float* u, int ldu, const void* w, const void* bias, int w_dtype,
+                        int taps, float* state, const int* token_slot, void* y, int ldy,
+                        int y_dtype, int act, int n_tokens, int C, hipStream_t stream);
 // The state after the step: the last taps - 1 of (the state, then the step's inputs).
 int hal_short_conv_carry(const float* u, int ldu, float* state, int taps, const int* seg_q_start,
                          const int* seg_q_len, const int* token_slot, int n_segs, int C,

@@ -41,6 +41,55 @@ __global__ void short_conv_kernel(const float* __restrict__ u, int ldu, const vo
   y[(size_t)t * ldy + c] = from_f32<TY>(acc);
 }
 
+// A step in which every segment is one token (decoding): the convolution and the carry in
+// one kernel; a thread owns its (request, channel) and moves the carried inputs one on.
+template <typename TY>
+__global__ void short_conv_step_kernel(const float* __restrict__ u, int ldu, const void* __restrict__ w,
+                                       const void* __restrict__ bias, int w_dtype, int taps,
+                                       float* __restrict__ state, const int* __restrict__ token_slot,
+                                       TY* __restrict__ y, int ldy, int act, int C) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int t = blockIdx.x;
+  if (c >= C) return;
+  float* st = state + (size_t)token_slot[t] * (taps - 1) * C + c;
+  const float x = u[(size_t)t * ldu + c];
+  float acc = bias ? load_as_f32(bias, w_dtype, c) : 0.f;
+  float old[CONV_MAX_TAPS];
+#pragma unroll
+  for (int j = 0; j < CONV_MAX_TAPS - 1; ++j)
+    if (j < taps - 1) old[j] = st[(size_t)j * C];
+#pragma unroll
+  for (int j = 0; j < CONV_MAX_TAPS - 1; ++j) {
+    if (j < taps - 1) {
+      acc = fmaf(load_as_f32(w, w_dtype, (size_t)c * taps + j), old[j], acc);
+      st[(size_t)j * C] = j + 1 < taps - 1 ? old[j + 1] : x;
+    }
+  }
+  acc = fmaf(load_as_f32(w, w_dtype, (size_t)c * taps + taps - 1), x, acc);
+  if (act == 1) acc = silu_f32(acc);
+  y[(size_t)t * ldy + c] = from_f32<TY>(acc);
+}
+
+extern "C" int hal_short_conv_step(const float* u, int ldu, const void* w, const void* bias, int w_dtype, int taps,
+                                   float* state, const int* token_slot, void* y, int ldy, int y_dtype, int act,
+                                   int n_tokens, int C, hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && C > 0 && taps >= 1 && taps <= CONV_MAX_TAPS && ldu >= C && ldy >= C,
+              "hal_short_conv_step: bad sizes T=%d C=%d taps=%d", n_tokens, C, taps);
+  HAL_REQUIRE(y_dtype == HAL_F32 || y_dtype == HAL_BF16, "hal_short_conv_step: dtype %d", y_dtype);
+  HAL_REQUIRE(act == 0 || act == 1, "hal_short_conv_step: activation %d", act);
+  HAL_REQUIRE((C + 255) / 256 <= 65535, "hal_short_conv_step: %d channels exceed the grid limit", C);
+  if (n_tokens == 0) return 0;
+  dim3 grid(n_tokens, (C + 255) / 256);
+  if (y_dtype == HAL_F32)
+    hipLaunchKernelGGL(short_conv_step_kernel<float>, grid, dim3(256), 0, stream, u, ldu, w, bias, w_dtype, taps, state,
+                       token_slot, (float*)y, ldy, act, C);
+  else
+    hipLaunchKernelGGL(short_conv_step_kernel<bf16_t>, grid, dim3(256), 0, stream, u, ldu, w, bias, w_dtype, taps, state,
+                       token_slot, (bf16_t*)y, ldy, act, C);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
 extern "C" int hal_short_conv(const float* u, int ldu, const void* w, const void* bias, int w_dtype, int taps,
                               const float* state, const int* token_seg, const int* seg_q_start,
                               const int* token_slot, void* y, int ldy, int y_dtype, int act, int n_tokens, int C,

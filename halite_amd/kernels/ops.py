@@ -984,6 +984,35 @@ def short_conv(u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None,
     return y
 
 
+def short_conv_through(u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, state: torch.Tensor,
+                       ctx, out_dtype: torch.dtype, silu: bool = False) -> torch.Tensor:
+    """``short_conv`` and ``short_conv_carry`` for the step ``ctx``: the convolution's result,
+    and the state left as the next step finds it.  A step in which every request brings
+    one token takes one kernel for both."""
+    c, taps = weight.shape
+    n = u.shape[0]
+    if taps == 1:
+        return short_conv(u, weight, bias, state, ctx.token_seg, ctx.seg_q_start, ctx.token_slot, out_dtype, silu)
+    if n == ctx.n_segs:
+        lib = library.core_library()
+        _rows_f32(u, c, "short_conv")
+        _dev(weight, bias, state)
+        slot = ctx.token_slot
+        _dev(slot)
+        _i32(slot, "token_slot")
+        _need(state.dtype == torch.float32 and state.dim() == 3 and state.shape[1:] == (taps - 1, c), "short_conv: state rows")
+        _need(bias is None or (bias.shape == (c,) and bias.dtype == weight.dtype), "short_conv: bias")
+        _need(slot.numel() == n, "short_conv: one slot a token")
+        y = torch.empty((n, c), dtype=out_dtype, device=u.device)
+        _check(lib, lib.hal_short_conv_step(
+            _ptr(u), u.stride(0), _ptr(weight), _ptr(bias), dtype_code(weight.dtype), taps, _ptr(state), _ptr(slot),
+            _ptr(y), c, dtype_code(out_dtype), 1 if silu else 0, n, c, _stream()))
+        return y
+    y = short_conv(u, weight, bias, state, ctx.token_seg, ctx.seg_q_start, ctx.token_slot, out_dtype, silu)
+    short_conv_carry(u, state, ctx.seg_q_start, ctx.seg_q_len, ctx.token_slot)
+    return y
+
+
 def short_conv_carry(u: torch.Tensor, state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
                      token_slot: torch.Tensor) -> None:
     """After ``short_conv``: every request's state becomes the last ``taps - 1`` of (its

@@ -199,10 +199,7 @@ class NormedAttention(Mixer):
         n, D = x.shape[0], self.head_dim
         a = ops.linear(x, self.w_qkv, out_dtype=torch.float32, tiled=self.t_qkv)
         if p.conv_taps is not None and p.conv_taps > 1:
-            state = run.state["conv"]
-            u = a
-            a = ops.short_conv(u, self.w_conv, None, state, ctx.token_seg, ctx.seg_q_start, ctx.token_slot, torch.float32)
-            ops.short_conv_carry(u, state, ctx.seg_q_start, ctx.seg_q_len, ctx.token_slot)
+            a = ops.short_conv_through(a, self.w_conv, None, run.state["conv"], ctx, torch.float32)
         elif p.conv_taps == 1:
             a = ops.short_conv(a, self.w_conv, None, a.new_zeros((1, 0, a.shape[1])), ctx.token_seg, ctx.seg_q_start,
                                ctx.token_slot, torch.float32)

@@ -117,10 +117,7 @@ class StateSpace(Mixer):
         u = a[:, inner : inner + self.conv_channels]
         dt_raw = a[:, inner + self.conv_channels :]
         conv_state = run.state["conv"] if p.conv_taps > 1 else a.new_zeros((1, 0, self.conv_channels))
-        xbc = ops.short_conv(u, self.conv_weight, self.conv_bias, conv_state, ctx.token_seg, ctx.seg_q_start,
-                             ctx.token_slot, x.dtype, silu=True)
-        if p.conv_taps > 1:
-            ops.short_conv_carry(u, conv_state, ctx.seg_q_start, ctx.seg_q_len, ctx.token_slot)
+        xbc = ops.short_conv_through(u, self.conv_weight, self.conv_bias, conv_state, ctx, x.dtype, silu=True)
         cut = ctx.has_array(f"scan_chunks_{SCAN_CHUNK}")
         y = ops.ssd_scan(xbc, dt_raw, self.dt_bias, self.A_log, self.D, run.state["state"], ctx.seg_q_start,
                          ctx.seg_q_len, ctx.token_slot, p.groups,

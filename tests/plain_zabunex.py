@@ -360,8 +360,8 @@ ZAB_B_BIAS = {1: 10}
 # convolution of one tap and one of five, a chunk of exactly a page, a single bias row per
 # distance up to the table's half
 ZAB_C = model_cfg(40, 199, [
-    attention_layer(3, 3, 20, 0.22, 100, 0.5, 64, ff=52),
-    parallel_layer(left_cfg(3, 3, 12, 20, 0.29, 5, 16, 4, base=1.0e6, factor=8.0), right_cfg(5, 12, 24, 5, 1, 3), 0.6, 1.1, ff=36),
+    attention_layer(3, 3, 20, 0.22, 100, 0.45, 48, ff=52),
+    parallel_layer(left_cfg(3, 3, 12, 20, 0.29, 5, 16, 4, base=2.0e5, factor=6.0), right_cfg(5, 12, 24, 5, 1, 3), 0.55, 1.25, ff=36),
     attention_layer(2, 1, 12, 0.3, 9, 0.0, 5),
 ])
 ZAB_C_BIAS = {0: 6, 2: 16}

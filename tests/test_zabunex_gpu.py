@@ -6,6 +6,8 @@ back, at the first positions, and on both sides of a chunk's edge where that edg
 a page's, long decoding beside requests that come and go, the stream after every layer,
 and greedy generation through the engine's entry point."""
 
+from types import SimpleNamespace
+
 import pytest
 import torch
 
@@ -163,30 +165,30 @@ def test_short_convolution_in_steps(gpu, taps, act):
     taps, many), in slots that are not in order; the carried inputs make the steps equal to
     the whole sequences.  A slot that is zeroed serves a new request."""
     C = 70
-    seqs = {2: rand(40, 3 + C, seed=10), 0: rand(23, 3 + C, seed=11)}
+    seqs = {2: rand(41, 3 + C, seed=10), 0: rand(24, 3 + C, seed=11)}
     w, b = rand(C, taps, seed=12, scale=0.5), rand(C, seed=13)
     want = {s: P.short_convolution(u[:, 3:].to(F), w.to(F), b.to(F)) for s, u in seqs.items()}
     if act:
         want = {s: P.silu(y) for s, y in want.items()}
     state = torch.full((4, taps - 1, C), float("nan"), device=gpu)
     state[0].zero_(), state[2].zero_()
-    plan = [({2: 1, 0: 2}), ({2: 2}), ({0: 1, 2: 30}), ({2: 7, 0: 20})]
+    # (a step of single tokens alone takes the kernel that convolves and carries at once)
+    plan = [({2: 1, 0: 2}), ({2: 2}), ({0: 1, 2: 1}), ({0: 1, 2: 30}), ({2: 7, 0: 20})]
     at = {2: 0, 0: 0}
     for step in plan:
         slots = list(step)
         cuts = [step[s] for s in slots]
         u = torch.cat([seqs[s][at[s] : at[s] + step[s]] for s in slots]).to(gpu)
         seg, starts, lens, slot = step_arrays(gpu, cuts, slots)
-        y = ops.short_conv(u[:, 3:], w.to(gpu), b.to(gpu), state, seg, starts, slot, torch.float32, silu=act).cpu()
-        if taps > 1:
-            ops.short_conv_carry(u[:, 3:], state, starts, lens, slot)
+        step_ctx = SimpleNamespace(token_seg=seg, seg_q_start=starts, seg_q_len=lens, token_slot=slot, n_segs=len(cuts))
+        y = ops.short_conv_through(u[:, 3:], w.to(gpu), b.to(gpu), state, step_ctx, torch.float32, silu=act).cpu()
         r = 0
         for s in slots:
             ref = want[s][at[s] : at[s] + step[s]]
             assert float((y[r : r + step[s]] - ref).abs().max()) < 1e-5, (taps, s, at[s])
             r += step[s]
             at[s] += step[s]
-    assert at == {2: 40, 0: 23}
+    assert at == {2: 41, 0: 24}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
