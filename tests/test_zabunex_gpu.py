@@ -518,3 +518,71 @@ def test_greedy_generation_through_the_engine(folders, name, dtype):
                 assert gap < (1e-4 if dtype == "float32" else 0.05), f"request {r.id} token {step}: {tok} for {best}, gap {gap}"
             ids.append(tok)
         assert len(r.output_ids[0]) == 12
+
+
+# -- the programs: generation from the command line, the random-weights mode, trace replay -----
+
+
+def test_command_line_and_replay_program(folders, tmp_path):
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder, _, _, weights = folders[("A", "float32")]
+    cfg = P.ZAB_A
+    cmd = [sys.executable, os.path.join(root, "bin", "halite_generate"), "--model", folder, "--prompt-ids", "5,17,3,90,9",
+           "sampling.temperature=0", "sampling.max_new_tokens=5", "model.dtype=float32", "server.kv_cache_num_tokens=256"]
+    proc = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    rec = json.loads(proc.stdout.strip().split("\n")[-1])
+    ids = [5, 17, 3, 90, 9]
+    for tok in rec["output_ids"][0]:
+        assert tok == int(torch.argmax(plain_logits(cfg, weights, ids)[-1]))
+        ids.append(tok)
+    assert len(ids) == 10
+    # the random-weights mode: a configuration without tensors states the rows of its bias
+    # tables; the folder it writes holds the design's own keys, and the engine reads the rows
+    # back from the tensors
+    stated = json.loads(json.dumps(P.ZAB_C))
+    for i, n in P.ZAB_C_BIAS.items():
+        stated["layers"][i]["mixer"]["bias_buckets"] = n
+    cfgfile, out = tmp_path / "c.json", tmp_path / "rand"
+    cfgfile.write_text(json.dumps(stated))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "halite_make_random_model"), "--config", str(cfgfile),
+                           "--out", str(out), "--seed", "3", "--dtype", "bfloat16", "--std", "0.1"], capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "bias_buckets" not in (out / "config.json").read_text()
+    # the replay program on that folder: a prompt in two portions and a decoded token, beside a
+    # second request; two slots, so the third request takes the one that was freed
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": [1, 2, 3, 4, 5], "want": [4]}, {"id": "b", "tokens": [7], "want": [0]}], "end": ["b"]},
+        {"step": 1, "entries": [{"id": "a", "tokens": [6, 7], "want": []}, {"id": "c", "tokens": [9, 8], "want": [1]}], "end": ["c"]},
+        {"step": 2, "entries": [{"id": "a", "tokens": [8], "want": [0]}], "end": ["a"]},
+    ]
+    logits = tmp_path / "logits"
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(out), "--dtype", "float32",
+                           "--out", str(logits), "--max-tokens", "128", "--slots", "2"],
+                          input="\n".join(json.dumps(s) for s in steps) + "\n", cwd=root, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.split("\n") if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    from safetensors.torch import load_file
+
+    stored = {k: v.float() for k, v in load_file(str(out / "model.safetensors")).items()}
+    want = plain_logits(P.ZAB_C, stored, [1, 2, 3, 4, 5, 6, 7, 8])
+    got0 = torch.from_numpy(np.fromfile(logits / "0.f32", dtype="<f4").reshape(2, -1))
+    got1 = torch.from_numpy(np.fromfile(logits / "1.f32", dtype="<f4").reshape(1, -1))
+    got2 = torch.from_numpy(np.fromfile(logits / "2.f32", dtype="<f4").reshape(1, -1))
+    scale = max(1.0, float(want.abs().max()))
+    assert float((got0[0] - want[4]).abs().max()) < 5e-5 * scale and float((got2[0] - want[7]).abs().max()) < 5e-5 * scale
+    assert float((got0[1] - plain_logits(P.ZAB_C, stored, [7])[0]).abs().max()) < 5e-5 * scale
+    assert float((got1[0] - plain_logits(P.ZAB_C, stored, [9, 8])[1]).abs().max()) < 5e-5 * scale
+    # a third live request has no slot
+    steps[0]["entries"].append({"id": "x", "tokens": [3], "want": []})
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(out), "--dtype", "float32",
+                           "--out", str(logits), "--max-tokens", "128", "--slots", "2"],
+                          input=json.dumps(steps[0]) + "\n", cwd=root, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 1 and "slots" in proc.stderr
