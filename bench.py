@@ -363,12 +363,13 @@ def llama_work(c, n_layers, tokens, batch=0, kv_tokens=0) -> dict:
 
 # Layers of the Zabunex design at two sizes that resemble served models: three layers of the
 # attention with a bias by distance and one of the chunked attention beside the state-space
-# mixer to every four, as many weights in the feed-forward's two matrices as in the three of
-# the Llama layer beside it (same width, heads, head size and grouping).
+# mixer to every four, a feed-forward of four times the width, and beside it a Llama layer of
+# the same width, heads, head size and grouping whose feed-forward's three matrices hold as
+# many weights as those two.
 ZABUNEX_SIZES = {
-    "2048-wide": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=12288, llama_ff=8192, chunk=1024, bias_max=128,
+    "2048-wide": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=8192, llama_ff=5504, chunk=1024, bias_max=128,
                       ssm_heads=32, ssm_dim=64, state=128, groups=8),
-    "4096-wide": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=21504, llama_ff=14336, chunk=1024, bias_max=128,
+    "4096-wide": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=16384, llama_ff=11008, chunk=1024, bias_max=128,
                       ssm_heads=64, ssm_dim=64, state=128, groups=8),
 }
 
