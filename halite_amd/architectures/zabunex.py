@@ -105,8 +105,6 @@ def zabunex_weight_map(cfg: ZabunexConfig) -> dict[str, str | None]:
         else:
             for theirs, ours in _LEFT_TENSORS:
                 table[f"{src}mix.left.{theirs}"] = f"{dst}mixer.left.{ours}"
-            if layer.mixer.left.conv == 1:
-                pass  # (a convolution of one tap is still a tensor of the folder)
             for theirs, ours in _RIGHT_TENSORS:
                 table[f"{src}mix.right.{theirs}"] = f"{dst}mixer.right.{ours}"
         if layer.mlp is None:

@@ -11,6 +11,7 @@ from .registry import (
     register_architecture,
 )
 from .spec import LayerRun, LayerSpec, ModelSpec, PartSpec
+from .zabunex import ZabunexConfig
 
 __all__ = [
     "ARCHITECTURES",
@@ -25,6 +26,7 @@ __all__ = [
     "ModelSpec",
     "PartSpec",
     "ServerConfig",
+    "ZabunexConfig",
     "get_architecture",
     "parse_config",
     "parse_overrides",
