@@ -12,7 +12,18 @@ from __future__ import annotations
 
 from typing import Annotated, Literal, Union
 
-from pydantic import BaseModel, ConfigDict, Field, StrictInt, model_validator
+from pydantic import BaseModel, BeforeValidator, ConfigDict, Field, StrictInt, model_validator
+
+
+def _whole_number(v):
+    """A size that a writer stored as a float without a fraction (64.0) is that integer;
+    anything else goes to the strict check as it is."""
+    if isinstance(v, float) and v.is_integer():
+        return int(v)
+    return v
+
+
+Size = Annotated[StrictInt, BeforeValidator(_whole_number)]
 
 
 class _Keys(BaseModel):
@@ -26,18 +37,18 @@ class ZabunexNorm(_Keys):
 
 class ZabunexQueryTemperature(_Keys):
     coef: float
-    every: StrictInt = Field(gt=0)
+    every: Size = Field(gt=0)
 
 
 class ZabunexBiasedAttention(_Keys):
-    heads: StrictInt = Field(gt=0)
-    kv_heads: StrictInt = Field(gt=0)
-    dim: StrictInt = Field(gt=0)
-    vdim: StrictInt = Field(gt=0)
+    heads: Size = Field(gt=0)
+    kv_heads: Size = Field(gt=0)
+    dim: Size = Field(gt=0)
+    vdim: Size = Field(gt=0)
     scale: float = Field(gt=0)
-    bias_max: StrictInt = Field(gt=0)
+    bias_max: Size = Field(gt=0)
     q_temp: ZabunexQueryTemperature
-    bias_buckets: StrictInt | None = Field(default=None, gt=1)
+    bias_buckets: Size | None = Field(default=None, gt=1)
 
     @model_validator(mode="after")
     def _check(self):
@@ -54,21 +65,21 @@ class ZabunexRotationScaling(_Keys):
 
 class ZabunexRotation(_Keys):
     base: float = Field(gt=0)
-    dims: StrictInt = Field(gt=0)
+    dims: Size = Field(gt=0)
     scaling: ZabunexRotationScaling
 
 
 class ZabunexMask(_Keys):
-    size: StrictInt = Field(gt=0)
+    size: Size = Field(gt=0)
 
 
 class ZabunexChunkedAttention(_Keys):
-    heads: StrictInt = Field(gt=0)
-    kv_heads: StrictInt = Field(gt=0)
-    dim: StrictInt = Field(gt=0)
-    vdim: StrictInt = Field(gt=0)
+    heads: Size = Field(gt=0)
+    kv_heads: Size = Field(gt=0)
+    dim: Size = Field(gt=0)
+    vdim: Size = Field(gt=0)
     scale: float = Field(gt=0)
-    conv: StrictInt = Field(gt=0)
+    conv: Size = Field(gt=0)
     mask: ZabunexMask
     rot: ZabunexRotation
 
@@ -82,12 +93,12 @@ class ZabunexChunkedAttention(_Keys):
 
 
 class ZabunexStateSpace(_Keys):
-    heads: StrictInt = Field(gt=0)
-    vdim: StrictInt = Field(gt=0)
-    state: StrictInt = Field(gt=0)
-    groups: StrictInt = Field(gt=0)
-    conv: StrictInt = Field(gt=0)
-    norm_groups: StrictInt = Field(gt=0)
+    heads: Size = Field(gt=0)
+    vdim: Size = Field(gt=0)
+    state: Size = Field(gt=0)
+    groups: Size = Field(gt=0)
+    conv: Size = Field(gt=0)
+    norm_groups: Size = Field(gt=0)
 
 
 class ZabunexParallelMixer(_Keys):
@@ -99,7 +110,7 @@ class ZabunexParallelMixer(_Keys):
 
 class ZabunexDense(_Keys):
     kind: Literal["dense"]
-    ff: StrictInt = Field(gt=0)
+    ff: Size = Field(gt=0)
 
 
 class ZabunexAttentionLayer(_Keys):
@@ -123,11 +134,11 @@ class ZabunexConfig(BaseModel):
     model_config = ConfigDict(extra="ignore")
 
     architecture: Literal["Zabunex"]
-    vocab: StrictInt = Field(gt=0)
-    width: StrictInt = Field(gt=0)
+    vocab: Size = Field(gt=0)
+    width: Size = Field(gt=0)
     norm: ZabunexNorm
     layers: list[ZabunexLayer] = Field(min_length=1)
-    max_positions: StrictInt | None = Field(default=None, gt=0)
+    max_positions: Size | None = Field(default=None, gt=0)
     """Not a key of the design (a request may be as long as the cache allows); a folder may
     state it to bound the position tables."""
     stop_token_ids: tuple[int, ...] = ()

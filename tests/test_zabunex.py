@@ -57,6 +57,17 @@ def test_configurations_that_are_refused(bad):
         parse_config(cfg)
 
 
+def test_sizes_written_as_floats_without_a_fraction():
+    cfg = json.loads(json.dumps(P.ZAB_A))
+    cfg["width"], cfg["layers"][0]["mixer"]["bias_max"], cfg["layers"][1]["mixer"]["left"]["mask"]["size"] = 64.0, 40.0, 24.0
+    _, parsed = parse_config(cfg)
+    assert (parsed.width, parsed.layers[0].mixer.bias_max, parsed.layers[1].mixer.left.mask.size) == (64, 40, 24)
+    assert all(type(v) is int for v in (parsed.width, parsed.layers[0].mixer.bias_max))
+    cfg["width"] = 64.5
+    with pytest.raises(ConfigError):
+        parse_config(cfg)
+
+
 @pytest.mark.parametrize("name", list(CONFIGS))
 def test_the_model_as_data_and_its_tensors(name, tmp_path):
     cfg, rows = CONFIGS[name]
